@@ -1,6 +1,8 @@
-"""Feed-forward sublayers that are not gated linear units: a dense layer
-with the xIELU activation, and a mixture of small experts chosen by a
-per-token-id table (no learned router at run time)."""
+"""Feed-forward sublayers beyond the SwiGLU of the Llama family: a dense
+layer with the xIELU activation, a mixture of small experts chosen by a
+per-token-id table (no learned router at run time), a gated dense layer with
+the tanh form of gelu, and a mixture of clamped gated experts chosen by a
+learned router."""
 from __future__ import annotations
 
 import math
@@ -19,6 +21,7 @@ class FFCfg:
     ff: int                  # hidden size (of one expert for "moe")
     experts: int = 0
     top: int = 0
+    limit: float = 0.0       # clamp of the routed experts' gate and up
 
 
 def _softplus(x: float) -> float:
@@ -134,4 +137,135 @@ class TableMoE(nn.Module):
             done[at: at + n] = ops.linear(a, self.w_down[e])
             at += n
         ops.combine_rows(out, done, inv)
+        return out
+
+
+class GeluGatedFF(nn.Module):
+    """down(gelu_tanh(gate h) * (up h)); gate and up are one fused GEMM."""
+
+    def __init__(self, f: FFCfg, width: int, t: Dict[str, torch.Tensor],
+                 p: str, device, dtype):
+        super().__init__()
+        from kukeon_amd.models.mixers import fuse_rows
+        self.ff = f.ff
+        self.col, self.w_in = fuse_rows(
+            [("gate", t[p + "gate"]), ("up", t[p + "up"])], width, dtype,
+            device)
+        self.w_down = nn.Parameter(t[p + "down"].to(device=device,
+                                                    dtype=dtype)
+                                   .contiguous(), requires_grad=False)
+
+    @staticmethod
+    def tensor_shapes(f: FFCfg, width: int, vocab: int) -> Dict[str, tuple]:
+        return {"gate": (f.ff, width), "up": (f.ff, width),
+                "down": (width, f.ff)}
+
+    def forward(self, h: torch.Tensor, ids: torch.Tensor,
+                meta=None) -> torch.Tensor:
+        z = ops.linear(h, self.w_in)
+        a = torch.empty(h.shape[0], self.ff, dtype=h.dtype, device=h.device)
+        c = self.col
+        ops.gelu_glu(a, z[:, c["gate"]: c["gate"] + self.ff],
+                     z[:, c["up"]: c["up"] + self.ff])
+        return ops.linear(a, self.w_down)
+
+
+class RoutedMoE(nn.Module):
+    """`experts` small gated feed-forward layers without biases; a token
+    uses the `top` experts with the largest router logits, weighted by the
+    softmax over those logits only. Expert: g = min(gate h, limit),
+    u = clamp(up h, +-limit), y = g sigmoid(1.702 g) (u + 1), out = down y.
+    The router runs in fp32. Weights are stacked [E, 2 ff', W] (gate rows,
+    then up rows, each padded to a multiple of 8) and [E, W, ff].
+
+    Two forms behind one call. Few rows (decode steps; nothing leaves the
+    device, so the step can sit in a captured graph): every expert runs on
+    every row as one batched GEMM pair — a batch of a few dozen rows
+    touches nearly every expert anyway, so the weights stream once — and
+    the fold picks each row's chosen results. Many rows (prompt portions):
+    the (row, expert) pairs are sorted by expert, the group sizes come to
+    the host, and each expert runs plain GEMMs over its contiguous rows."""
+
+    sorted_min_rows = 64
+    alpha = 1.702
+
+    def __init__(self, f: FFCfg, width: int, t: Dict[str, torch.Tensor],
+                 p: str, device, dtype):
+        super().__init__()
+        if not (0 < f.top <= f.experts):
+            raise ValueError(f"{p}: top must be within 1 .. experts")
+        self.f = f
+        dev = dict(device=device, dtype=dtype)
+        pad = (f.ff + 7) // 8 * 8
+        self.up_col = pad
+        gu = torch.zeros(f.experts, 2 * pad, width, **dev)
+        for e in range(f.experts):
+            gu[e, :f.ff] = t[p + f"e{e}.gate"].to(**dev)
+            gu[e, pad: pad + f.ff] = t[p + f"e{e}.up"].to(**dev)
+        self.w_gu = nn.Parameter(gu.contiguous(), requires_grad=False)
+        self.w_down = nn.Parameter(torch.stack(
+            [t[p + f"e{e}.down"] for e in range(f.experts)]).to(**dev)
+            .contiguous(), requires_grad=False)
+        self.w_router = t[p + "router"].to(device=device,
+                                           dtype=torch.float32).contiguous()
+
+    @staticmethod
+    def tensor_shapes(f: FFCfg, width: int, vocab: int) -> Dict[str, tuple]:
+        out = {"router": (f.experts, width)}
+        for e in range(f.experts):
+            out[f"e{e}.gate"] = (f.ff, width)
+            out[f"e{e}.up"] = (f.ff, width)
+            out[f"e{e}.down"] = (width, f.ff)
+        return out
+
+    def forward(self, h: torch.Tensor, ids: torch.Tensor,
+                meta=None) -> torch.Tensor:
+        f = self.f
+        T, W = h.shape
+        logits = torch.nn.functional.linear(h.float(), self.w_router)
+        idx = torch.empty(T, f.top, dtype=torch.int32, device=h.device)
+        wts = torch.empty(T, f.top, dtype=torch.float32, device=h.device)
+        out = torch.empty_like(h)
+        on_host = getattr(meta, "host_ids", None) is not None
+        if on_host and T >= self.sorted_min_rows:
+            ops.router_topk(idx, wts, logits, f.top, 0)
+            return self._forward_sorted(out, h, idx, wts)
+        # every expert over every row; idx names rows of the [E*T, W] result
+        ops.router_topk(idx, wts, logits, f.top, T)
+        E, ff = f.experts, f.ff
+        z = torch.bmm(h.unsqueeze(0).expand(E, T, W),
+                      self.w_gu.transpose(1, 2)).view(E * T, -1)
+        a = torch.empty(E * T, ff, dtype=h.dtype, device=h.device)
+        ops.clamp_glu(a, z[:, :ff], z[:, self.up_col: self.up_col + ff],
+                      None, None, f.limit, self.alpha, 1.0)
+        y = torch.bmm(a.view(E, T, ff), self.w_down.transpose(1, 2))
+        ops.combine_rows_weighted(out, y.view(E * T, W), idx, wts)
+        return out
+
+    def _forward_sorted(self, out, h, idx, wts) -> torch.Tensor:
+        f = self.f
+        T, W = h.shape
+        E, ff, top = f.experts, f.ff, f.top
+        flat = idx.view(-1).long()
+        order = torch.argsort(flat, stable=True)
+        counts = torch.bincount(flat, minlength=E).tolist()  # host sync
+        inv = torch.empty_like(order)
+        inv[order] = torch.arange(order.numel(), device=h.device)
+        rows = torch.empty(T * top, W, dtype=h.dtype, device=h.device)
+        ops.gather_rows(rows, h, (order // top).to(torch.int32))
+        done = torch.empty_like(rows)
+        a = torch.empty(T * top, ff, dtype=h.dtype, device=h.device)
+        at = 0
+        for e in range(E):
+            n = counts[e]
+            if n == 0:
+                continue
+            z = ops.linear(rows[at: at + n], self.w_gu[e])
+            ops.clamp_glu(a[at: at + n], z[:, :ff],
+                          z[:, self.up_col: self.up_col + ff], None, None,
+                          f.limit, self.alpha, 1.0)
+            done[at: at + n] = ops.linear(a[at: at + n], self.w_down[e])
+            at += n
+        ops.combine_rows_weighted(out, done, inv.view(T, top)
+                                  .to(torch.int32), wts)
         return out

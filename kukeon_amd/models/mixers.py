@@ -1,9 +1,11 @@
 """Sequence mixers that carry their own kind of memory: a selective
-state-space mixer (fixed-size recurrent state per sequence) and a latent
-attention mixer (one low-rank row per token in the paged cache). Both take
-the normed layer input [T, W] of a packed batch plus the engine's row maps
-and return the mixer output [T, W]; all sizes and constants are arguments,
-so any model family can stack them.
+state-space mixer (fixed-size recurrent state per sequence), a latent
+attention mixer (one low-rank row per token in the paged cache), a
+grouped-query attention mixer with chunk-local keys and capped scores, and a
+linear-attention mixer with a fixed decay per head (a state matrix per
+sequence). All take the layer input [T, W] of a packed batch plus the
+engine's row maps and return the mixer output [T, W]; all sizes and constants
+are arguments, so any model family can stack them.
 """
 from __future__ import annotations
 
@@ -113,7 +115,8 @@ class StateSpaceMixer(nn.Module):
         m = self.m
         return [(m.conv - 1, m.conv_channels), (m.heads, m.vdim, m.state)]
 
-    def forward(self, h: torch.Tensor, cache, state, meta) -> torch.Tensor:
+    def forward(self, h: torch.Tensor, cache, state, meta,
+                cache_v=None) -> torch.Tensor:
         m = self.m
         T = h.shape[0]
         conv_state, ssm_state = state
@@ -153,6 +156,22 @@ class LatentAttnCfg:
     window: int              # position i sees i-window+1 .. i (0: all)
     rot_dims: int            # leading entries of the rotated part that turn
     rot_base: float
+    # "pairs": entries (2i, 2i+1) turn together; "half": entry i turns with
+    # entry i + rot_dims/2
+    rot_layout: str = "pairs"
+    # "head": one gate per head (g [H, W]); "element": one per output entry
+    # (g [H*vdim, W])
+    gate: str = "head"
+
+
+def _pairs_from_half(dims: int, n: int) -> torch.Tensor:
+    """Row order that turns the half layout of a rotated part of n entries
+    into the pair layout: new[2i] = old[i], new[2i+1] = old[i + dims/2]."""
+    half = dims // 2
+    order = []
+    for i in range(half):
+        order += [i, i + half]
+    return torch.tensor(order + list(range(dims, n)), dtype=torch.long)
 
 
 class LatentAttention(nn.Module):
@@ -166,31 +185,55 @@ class LatentAttention(nn.Module):
         out_h(i)      = W_uv_h  sum_j softmax_j(score_h)(i, j) c(j)
 
     so the kernel reads each cache row once for all heads. Queries pass
-    their own normed latent (q_rank). A sliding window bounds the keys, and
-    every head's output is scaled by sigmoid of a gate projected from the
-    mixer's input.
+    their own normed latent (q_rank), or come straight from the input when
+    q_rank is 0. A sliding window may bound the keys, and the output is
+    scaled by sigmoid of a gate projected from the mixer's input, per head
+    or per entry.
 
-    Tensors (prefix p): dq [q_rank, W], dq.norm, uq [H*(dim+rot_dim), q_rank],
-    dkv [kv_rank+rot_dim, W], dkv.norm, uk [H*dim, kv_rank],
-    uv [H*vdim, kv_rank], g [H, W], o [W, H*vdim]."""
+    The kernels turn pairs (2i, 2i+1). A checkpoint in the half layout
+    (entry i with i + rot_dims/2) has the rows of the rotated parts of its
+    query and key projections reordered at load; a score is a dot product
+    over those rows, so only its order of summation changes.
+
+    Tensors (prefix p): dq [q_rank, W], dq.norm, uq [H*(dim+rot_dim), q_rank]
+    (or q [H*(dim+rot_dim), W] when q_rank is 0), dkv [kv_rank+rot_dim, W],
+    dkv.norm, uk [H*dim, kv_rank], uv [H*vdim, kv_rank], g [H or H*vdim, W],
+    o [W, H*vdim]."""
 
     def __init__(self, m: LatentAttnCfg, width: int, eps: float,
                  t: Dict[str, torch.Tensor], p: str, device, dtype):
         super().__init__()
         if m.rot_dims % 2 or m.rot_dims > m.rot_dim:
             raise ValueError(f"{p}: bad rotary dims")
+        if m.rot_layout not in ("pairs", "half"):
+            raise ValueError(f"{p}: unknown rotary layout {m.rot_layout!r}")
+        if m.gate not in ("head", "element"):
+            raise ValueError(f"{p}: unknown gate kind {m.gate!r}")
         self.m = m
         self.eps = eps
+        H, R = m.heads, m.kv_rank
+        hd = m.dim + m.rot_dim
+        w_q = t[p + ("uq" if m.q_rank else "q")]
+        w_dkv = t[p + "dkv"]
+        if m.rot_layout == "half":
+            order = _pairs_from_half(m.rot_dims, m.rot_dim)
+            w_q = w_q.view(H, hd, -1)
+            w_q = torch.cat([w_q[:, :m.dim], w_q[:, m.dim:][:, order]],
+                            1).reshape(H * hd, -1)
+            w_dkv = torch.cat([w_dkv[:R], w_dkv[R:][order]], 0)
+        first = ("q", t[p + "dq"] if m.q_rank else w_q)
         self.col, self.w_down = fuse_rows(
-            [("q", t[p + "dq"]), ("kv", t[p + "dkv"]), ("g", t[p + "g"])],
-            width, dtype, device)
+            [first, ("kv", w_dkv), ("g", t[p + "g"])], width, dtype, device)
         f32 = dict(device=device, dtype=torch.float32)
-        self.q_norm = t[p + "dq.norm"].to(**f32).contiguous()
+        self.q_norm = (t[p + "dq.norm"].to(**f32).contiguous() if m.q_rank
+                       else torch.empty(0, **f32))
         self.kv_norm = t[p + "dkv.norm"].to(**f32).contiguous()
         dev = dict(device=device, dtype=dtype)
-        self.w_uq = nn.Parameter(t[p + "uq"].to(**dev).contiguous(),
-                                 requires_grad=False)
-        H, R = m.heads, m.kv_rank
+        self.w_uq = None
+        if m.q_rank:
+            self.w_uq = nn.Parameter(w_q.to(**dev).contiguous(),
+                                     requires_grad=False)
+        self.gate_cols = H if m.gate == "head" else H * m.vdim
         # [H, dim, R]: q_abs_h = q_h W_uk_h;  [H, R, vdim]: o_h = l_h W_uv_h^T
         self.w_uk = nn.Parameter(t[p + "uk"].to(**dev).view(H, m.dim, R)
                                  .contiguous(), requires_grad=False)
@@ -204,12 +247,17 @@ class LatentAttention(nn.Module):
     @staticmethod
     def tensor_shapes(m: LatentAttnCfg, width: int) -> Dict[str, tuple]:
         H = m.heads
-        return {"dq": (m.q_rank, width), "dq.norm": (m.q_rank,),
-                "uq": (H * (m.dim + m.rot_dim), m.q_rank),
-                "dkv": (m.kv_rank + m.rot_dim, width),
-                "dkv.norm": (m.kv_rank,), "uk": (H * m.dim, m.kv_rank),
-                "uv": (H * m.vdim, m.kv_rank), "g": (H, width),
-                "o": (width, H * m.vdim)}
+        out = {"dkv": (m.kv_rank + m.rot_dim, width),
+               "dkv.norm": (m.kv_rank,), "uk": (H * m.dim, m.kv_rank),
+               "uv": (H * m.vdim, m.kv_rank),
+               "g": (H if m.gate == "head" else H * m.vdim, width),
+               "o": (width, H * m.vdim)}
+        if m.q_rank:
+            out.update({"dq": (m.q_rank, width), "dq.norm": (m.q_rank,),
+                        "uq": (H * (m.dim + m.rot_dim), m.q_rank)})
+        else:
+            out["q"] = (H * (m.dim + m.rot_dim), width)
+        return out
 
     def kv_spec(self) -> Optional[LayerKVSpec]:
         return LayerKVSpec(1, self.m.kv_rank + self.m.rot_dim, 0)
@@ -217,17 +265,22 @@ class LatentAttention(nn.Module):
     def state_shape(self):
         return None
 
-    def forward(self, h: torch.Tensor, cache, state, meta) -> torch.Tensor:
+    def forward(self, h: torch.Tensor, cache, state, meta,
+                cache_v=None) -> torch.Tensor:
         m = self.m
         T = h.shape[0]
         H, R = m.heads, m.kv_rank
+        hd = m.dim + m.rot_dim
         proj = ops.linear(h, self.w_down)
         cq = torch.empty(T, m.q_rank, dtype=h.dtype, device=h.device)
         ops.latent_kv_append(cq, cache, proj, self.col["q"], self.col["kv"],
                              self.q_norm, self.kv_norm, self.eps, self.cs,
                              meta.positions, meta.row_seq, meta.block_table)
-        q = ops.linear(cq, self.w_uq)                  # [T, H*(dim+rot)]
-        q_n = q.view(T, H, m.dim + m.rot_dim)[:, :, :m.dim].transpose(0, 1)
+        if m.q_rank:
+            q = ops.linear(cq, self.w_uq)              # [T, H*(dim+rot)]
+        else:
+            q = proj[:, self.col["q"]: self.col["q"] + H * hd]
+        q_n = q.unflatten(1, (H, hd))[:, :, :m.dim].transpose(0, 1)
         q_abs = torch.bmm(q_n, self.w_uk)              # [H, T, R]
         lat = torch.empty(H, T, R, dtype=h.dtype, device=h.device)
         ops.latent_attention(lat, q_abs, q, cache, self.cs, meta.positions,
@@ -235,5 +288,156 @@ class LatentAttention(nn.Module):
                              m.rot_dim, m.window, m.scale)
         o = torch.bmm(lat, self.w_uv)                  # [H, T, vdim]
         og = torch.empty(T, H * m.vdim, dtype=h.dtype, device=h.device)
-        ops.head_gate(og, o, proj[:, self.col["g"]: self.col["g"] + H])
+        ops.head_gate(og, o, proj[:, self.col["g"]:
+                                  self.col["g"] + self.gate_cols])
         return ops.linear(og, self.w_o)
+
+
+# ---------------------------------------------------------------------------
+@dataclass
+class ChunkAttnCfg:
+    heads: int
+    kv_heads: int
+    dim: int
+    vdim: int
+    scale: float
+    softcap: float = 0.0     # scores become cap tanh(score / cap) (0: off)
+    chunk: int = 0           # keys of the query's own chunk only (0: all)
+    kv_from: Optional[int] = None    # read this earlier layer's pages
+
+
+class ChunkedAttention(nn.Module):
+    """Grouped-query softmax attention without positions in the scores.
+    Queries and keys are RMS-normed over their WHOLE projection (all heads
+    at once, one weight entry per row of the projection) before they are cut
+    into heads; scores are scaled, optionally capped with tanh, and position
+    i sees j <= i of its own chunk, floor(i / chunk) == floor(j / chunk).
+    A mixer with `kv_from` projects no keys or values and reads the pages
+    of that earlier layer with its own queries.
+
+    Tensors (prefix p): q [H*dim, W], q.norm [H*dim], o [W, H*vdim] and, for
+    a layer with pages of its own, k [G*dim, W], k.norm [G*dim],
+    v [G*vdim, W]."""
+
+    def __init__(self, m: ChunkAttnCfg, width: int, eps: float,
+                 t: Dict[str, torch.Tensor], p: str, device, dtype):
+        super().__init__()
+        if m.heads % m.kv_heads:
+            raise ValueError(f"{p}: heads not a multiple of kv_heads")
+        self.m = m
+        self.eps = eps
+        self.owns_kv = m.kv_from is None
+        segs = [("q", t[p + "q"])]
+        if self.owns_kv:
+            segs += [("k", t[p + "k"]), ("v", t[p + "v"])]
+        self.col, self.w_in = fuse_rows(segs, width, dtype, device)
+        f32 = dict(device=device, dtype=torch.float32)
+        self.q_norm = t[p + "q.norm"].to(**f32).contiguous()
+        self.k_norm = (t[p + "k.norm"].to(**f32).contiguous()
+                       if self.owns_kv else None)
+        self.w_o = nn.Parameter(t[p + "o"].to(device=device, dtype=dtype)
+                                .contiguous(), requires_grad=False)
+
+    @staticmethod
+    def tensor_shapes(m: ChunkAttnCfg, width: int) -> Dict[str, tuple]:
+        out = {"q": (m.heads * m.dim, width), "q.norm": (m.heads * m.dim,),
+               "o": (width, m.heads * m.vdim)}
+        if m.kv_from is None:
+            out.update({"k": (m.kv_heads * m.dim, width),
+                        "k.norm": (m.kv_heads * m.dim,),
+                        "v": (m.kv_heads * m.vdim, width)})
+        return out
+
+    def kv_spec(self) -> Optional[LayerKVSpec]:
+        return LayerKVSpec(self.m.kv_heads, self.m.dim, self.m.vdim,
+                           share_from=self.m.kv_from)
+
+    def state_shape(self):
+        return None
+
+    def forward(self, h: torch.Tensor, cache, state, meta,
+                cache_v=None) -> torch.Tensor:
+        m = self.m
+        T = h.shape[0]
+        proj = ops.linear(h, self.w_in)
+        q = torch.empty(T, m.heads * m.dim, dtype=h.dtype, device=h.device)
+        c = self.col
+        ops.qk_norm_append(q, cache if self.owns_kv else None,
+                           cache_v if self.owns_kv else None, proj, c["q"],
+                           c.get("k", 0), c.get("v", 0), self.q_norm,
+                           self.k_norm, self.eps, meta.positions,
+                           meta.row_seq, meta.block_table)
+        o = torch.empty(T, m.heads * m.vdim, dtype=h.dtype, device=h.device)
+        ops.chunk_attention(o, q, cache, cache_v, meta.positions,
+                            meta.row_seq, meta.block_table, m.heads, m.scale,
+                            m.softcap, m.chunk)
+        return ops.linear(o, self.w_o)
+
+
+# ---------------------------------------------------------------------------
+@dataclass
+class LightningCfg:
+    heads: int
+    dim: int
+    vdim: int
+    decay: tuple             # one factor per head
+
+
+class LightningMixer(nn.Module):
+    """Linear attention with a fixed decay per head. q, k and v are silu of
+    their projections, head by head; per head the state matrix follows
+    S_t = decay_h S_(t-1) + k_t v_t^T and the output is S_t^T q_t, with no
+    other scale. The heads' outputs are RMS-normed together, multiplied by
+    sigmoid of a gate projected from the mixer's input, and projected out.
+    The state (fp32, stored transposed as [H, vdim, dim]) lives in the
+    engine's state slots.
+
+    Tensors (prefix p): q, k [H*dim, W], v, g [H*vdim, W], norm [H*vdim],
+    o [W, H*vdim]."""
+
+    def __init__(self, m: LightningCfg, width: int, eps: float,
+                 t: Dict[str, torch.Tensor], p: str, device, dtype):
+        super().__init__()
+        if len(m.decay) != m.heads:
+            raise ValueError(f"{p}: one decay per head is needed")
+        self.m = m
+        self.eps = eps
+        self.col, self.w_in = fuse_rows(
+            [("q", t[p + "q"]), ("k", t[p + "k"]), ("v", t[p + "v"]),
+             ("g", t[p + "g"])], width, dtype, device)
+        f32 = dict(device=device, dtype=torch.float32)
+        self.decay = torch.tensor([float(d) for d in m.decay],
+                                  dtype=torch.float64).to(**f32).contiguous()
+        self.norm_w = t[p + "norm"].to(**f32).contiguous()
+        self.w_o = nn.Parameter(t[p + "o"].to(device=device, dtype=dtype)
+                                .contiguous(), requires_grad=False)
+
+    @staticmethod
+    def tensor_shapes(m: LightningCfg, width: int) -> Dict[str, tuple]:
+        H = m.heads
+        return {"q": (H * m.dim, width), "k": (H * m.dim, width),
+                "v": (H * m.vdim, width), "g": (H * m.vdim, width),
+                "norm": (H * m.vdim,), "o": (width, H * m.vdim)}
+
+    def kv_spec(self) -> Optional[LayerKVSpec]:
+        return None
+
+    def state_shape(self):
+        # the slot holds S^T: a column of S is one contiguous run
+        return (self.m.heads, self.m.vdim, self.m.dim)
+
+    def forward(self, h: torch.Tensor, cache, state, meta,
+                cache_v=None) -> torch.Tensor:
+        m = self.m
+        T = h.shape[0]
+        inner = m.heads * m.vdim
+        proj = ops.linear(h, self.w_in)
+        c = self.col
+        y = torch.empty(T, inner, dtype=torch.float32, device=h.device)
+        ops.lightning_scan(y, proj, c["q"], c["k"], c["v"], self.decay, state,
+                           meta.positions, meta.cu_rows, meta.state_slots,
+                           m.heads, m.dim, m.vdim)
+        g = torch.empty(T, inner, dtype=h.dtype, device=h.device)
+        ops.gated_rmsnorm(g, y, proj[:, c["g"]: c["g"] + inner], self.norm_w,
+                          self.eps)
+        return ops.linear(g, self.w_o)

@@ -32,8 +32,14 @@ def _rasesun(cfg, device, **kw):
     return RasesunModel(cfg, device=device, **kw)
 
 
+def _dumovik(cfg, device, **kw):
+    from kukeon_amd.models.dumovik import DumovikModel
+    return DumovikModel(cfg, device=device, **kw)
+
+
 # family -> constructor(cfg, device, **kw)
 FAMILIES: Dict[str, Callable] = {
+    "dumovik": _dumovik,
     "llama": _llama,
     "mixtral": _mixtral,
     "lipedra": _lipedra,
@@ -44,6 +50,7 @@ FAMILIES: Dict[str, Callable] = {
 ARCHITECTURES: Dict[str, str] = {
     "Lipedra": "lipedra",
     "Rasesun": "rasesun",
+    "Dumovik": "dumovik",
 }
 
 
@@ -54,6 +61,7 @@ OP_GROUPS: Dict[str, tuple] = {
     "mixtral": ("core",),
     "lipedra": ("mix",),
     "rasesun": ("recur",),
+    "dumovik": ("hyb",),
 }
 
 
@@ -108,12 +116,33 @@ RASESUN_PRESETS = {
 }
 
 
+def _dumovik_preset(**kw):
+    def make():
+        from kukeon_amd.models.dumovik import dumovik_bench
+        return dumovik_bench(**kw)
+    return make
+
+
+# random-weight Dumovik stacks: periods of chunked attention, two linear
+# attention layers and latent attention at Llama-3-8B width, and a small one
+DUMOVIK_PRESETS = {
+    "dumovik-8b-like": _dumovik_preset(width=4096, layers=32, heads=32,
+                                       kv_heads=8, ff=14336, vocab=128256,
+                                       name="dumovik-8b-like"),
+    "tiny-dumovik": _dumovik_preset(width=128, layers=8, heads=2, kv_heads=1,
+                                    ff=256, vocab=384, chunk=24, experts=4,
+                                    name="tiny-dumovik"),
+}
+
+
 def preset_names():
     return sorted(list(MODEL_PRESETS) + list(LIPEDRA_PRESETS) +
-                  list(RASESUN_PRESETS))
+                  list(RASESUN_PRESETS) + list(DUMOVIK_PRESETS))
 
 
 def preset(name: str):
+    if name in DUMOVIK_PRESETS:
+        return DUMOVIK_PRESETS[name]()
     if name in LIPEDRA_PRESETS:
         return LIPEDRA_PRESETS[name]()
     if name in RASESUN_PRESETS:
@@ -139,5 +168,9 @@ def load_checkpoint(model_dir: str, device, dtype: str = "bf16"):
     if fam == "rasesun":
         from kukeon_amd.models.rasesun import RasesunModel
         return RasesunModel.from_checkpoint(model_dir, device=device,
+                                            dtype=dtype)
+    if fam == "dumovik":
+        from kukeon_amd.models.dumovik import DumovikModel
+        return DumovikModel.from_checkpoint(model_dir, device=device,
                                             dtype=dtype)
     raise ValueError(f"family {fam} has no checkpoint loader")

@@ -89,6 +89,58 @@ def _recur(t: torch.Tensor):
     return _C_recur
 
 
+_C_hyb = None
+_HYB_IMPORT_ERROR: Exception | None = None
+try:
+    from kukeon_amd import _C_hyb  # type: ignore
+except Exception as e:  # pragma: no cover
+    _HYB_IMPORT_ERROR = e
+
+
+def hyb_available() -> bool:
+    return _C_hyb is not None
+
+
+def _hyb(t: torch.Tensor):
+    """Kernel group of the hybrid stacks (output-side layer norm, chunked
+    attention, decayed linear attention, routed experts): native on a GPU
+    tensor (an error if the module is not built), fp32 references on CPU."""
+    global _C_hyb, _HYB_IMPORT_ERROR
+    if not t.is_cuda:
+        return reference
+    if _C_hyb is None:
+        try:
+            import importlib
+            _C_hyb = importlib.import_module("kukeon_amd._C_hyb")
+        except Exception as e:
+            _HYB_IMPORT_ERROR = e
+    if _C_hyb is None:
+        raise RuntimeError(
+            "kukeon_amd._C_hyb (gfx950 HIP extension) is not built but an "
+            "op was called on a CUDA device. Run `python -m "
+            f"kukeon_amd.ops.build hyb` (import error: {_HYB_IMPORT_ERROR})")
+    return _C_hyb
+
+
+def _shared(t: torch.Tensor, first, second):
+    """A kernel that two groups compile from the same source: whichever of
+    the two modules is built serves it (`first` preferred)."""
+    if not t.is_cuda:
+        return reference
+    key = (first, second)
+    mod = _SHARED_CHOICE.get(key)
+    if mod is None:
+        try:
+            mod = first(t)
+        except RuntimeError:
+            mod = second(t)
+        _SHARED_CHOICE[key] = mod
+    return mod
+
+
+_SHARED_CHOICE: dict = {}
+
+
 def _native():
     if _C is None:
         raise RuntimeError(
@@ -374,11 +426,10 @@ def residual_add_rmsnorm(x, a, bias, w, w_offset: float, eps: float,
 
 def clamp_glu(out, gate, up, bg, bu, limit: float, alpha: float = 1.702,
               up_shift: float = 1.0) -> None:
-    _mix(out).clamp_glu(out, gate, up,
-                        bg if bg is not None else _e(bu if bu is not None
-                                                     else out.float()),
-                        bu if bu is not None else _e(out.float()),
-                        limit, alpha, up_shift)
+    none = torch.empty(0, dtype=torch.float32, device=out.device)
+    _shared(out, _mix, _hyb).clamp_glu(
+        out, gate, up, bg if bg is not None else none,
+        bu if bu is not None else none, limit, alpha, up_shift)
 
 
 def conv_rope_append(q_out, k_cache, v_cache, proj, bias, cw, state, cs,
@@ -509,20 +560,21 @@ def gated_group_rmsnorm(out, y, z, w, groups: int, eps: float) -> None:
 def latent_kv_append(cq_out, cache, proj, q_col: int, kv_col: int, wq, wkv,
                      eps: float, cs, positions, row_seq,
                      block_table) -> None:
-    _recur(proj).latent_kv_append(cq_out, cache, proj, q_col, kv_col, wq,
-                                  wkv, eps, cs, positions, row_seq,
-                                  block_table)
+    _shared(proj, _recur, _hyb).latent_kv_append(
+        cq_out, cache, proj, q_col, kv_col, wq, wkv, eps, cs, positions,
+        row_seq, block_table)
 
 
 def latent_attention(out, q_abs, q, cache, cs, positions, row_seq,
                      block_table, H: int, dn: int, dr: int, window: int,
                      scale: float) -> None:
-    _recur(q).latent_attention(out, q_abs, q, cache, cs, positions, row_seq,
-                               block_table, H, dn, dr, window, scale)
+    _shared(q, _recur, _hyb).latent_attention(
+        out, q_abs, q, cache, cs, positions, row_seq, block_table, H, dn, dr,
+        window, scale)
 
 
 def head_gate(out, o, gate) -> None:
-    _recur(out).head_gate(out, o, gate)
+    _shared(out, _recur, _hyb).head_gate(out, o, gate)
 
 
 def xielu(out, z, ap: float, aq: float) -> None:
@@ -534,7 +586,7 @@ def table_moe(out, h, ids, table, w_up, w_down) -> None:
 
 
 def gather_rows(out, inp, row_map) -> None:
-    _recur(out).gather_rows(out, inp, row_map)
+    _shared(out, _recur, _hyb).gather_rows(out, inp, row_map)
 
 
 def relu_square_(x) -> None:
@@ -547,3 +599,60 @@ def combine_rows(out, inp, inv) -> None:
 
 def softcap_(logits, cap: float) -> None:
     _recur(logits).softcap_(logits, cap)
+
+
+# ---- hybrid group ----------------------------------------------------------
+def layernorm_residual(x, y, w, eps: float, out) -> None:
+    """x (fp32 residual, in place) += layernorm(y) * w (mean taken off, no
+    bias); out = x in the activation format."""
+    _hyb(x).layernorm_residual(x, y, w, eps, out)
+
+
+def layernorm(out, x, w, eps: float) -> None:
+    _hyb(x).layernorm(out, x, w, eps)
+
+
+def gelu_glu(out, gate, up) -> None:
+    """out = gelu_tanh(gate) * up; gate and up are views into one fused
+    projection."""
+    _hyb(out).gelu_glu(out, gate, up)
+
+
+def qk_norm_append(q_out, k_cache, v_cache, proj, q_col: int, k_col: int,
+                   v_col: int, wq, wk, eps: float, positions, row_seq,
+                   block_table) -> None:
+    """RMS norm over the WHOLE query projection (and the whole key
+    projection) of a row, then the key and value rows go to their page. A
+    layer that reads another layer's pages passes k_cache = None."""
+    if k_cache is None:
+        k_cache = v_cache = _e(proj)
+        wk = _e(wq)
+    _hyb(proj).qk_norm_append(q_out, k_cache, v_cache, proj, q_col, k_col,
+                              v_col, wq, wk, eps, positions, row_seq,
+                              block_table)
+
+
+def chunk_attention(out, q, k_cache, v_cache, positions, row_seq,
+                    block_table, H: int, scale: float, softcap: float,
+                    chunk: int) -> None:
+    _hyb(q).chunk_attention(out, q, k_cache, v_cache, positions, row_seq,
+                            block_table, H, scale, softcap, chunk)
+
+
+def lightning_scan(y, proj, q_col: int, k_col: int, v_col: int, decay, state,
+                   positions, cu_rows, state_slots, H: int, d: int,
+                   dv: int) -> None:
+    _hyb(proj).lightning_scan(y, proj, q_col, k_col, v_col, decay, state,
+                              positions, cu_rows, state_slots, H, d, dv)
+
+
+def gated_rmsnorm(out, y, gate, w, eps: float) -> None:
+    _hyb(out).gated_rmsnorm(out, y, gate, w, eps)
+
+
+def router_topk(idx, wts, logits, top: int, dense_rows: int = 0) -> None:
+    _hyb(logits).router_topk(idx, wts, logits, top, dense_rows)
+
+
+def combine_rows_weighted(out, inp, inv, wts) -> None:
+    _hyb(out).combine_rows_weighted(out, inp, inv, wts)

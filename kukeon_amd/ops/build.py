@@ -47,6 +47,22 @@ RECUR_SOURCES = [
     "bindings_recur.cpp",
 ]
 
+#   hyb -> kukeon_amd/_C_hyb.so   (output-side layer norm, chunk-local
+#                                  attention, decayed linear attention, gated
+#                                  activations, routed experts, latent
+#                                  attention)
+HYB_SOURCES = [
+    "layer_norm.hip",
+    "glu_clamp.hip",
+    "chunk_attn.hip",
+    "lightning.hip",
+    "routed_moe.hip",
+    "latent_attn.hip",
+    "recur_elem.hip",
+    "table_moe.hip",
+    "bindings_hyb.cpp",
+]
+
 SOURCES = [
     "rmsnorm.hip",
     "activation.hip",
@@ -78,6 +94,7 @@ GROUPS = {
     "core": ("_C", SOURCES),
     "mix": ("_C_mix", MIX_SOURCES),
     "recur": ("_C_recur", RECUR_SOURCES),
+    "hyb": ("_C_hyb", HYB_SOURCES),
 }
 
 

@@ -1,6 +1,7 @@
 // Small per-row and per-element kernels of the recurrent / latent group:
 //   gated_group_rmsnorm  out = rmsnorm_by_part(y * silu(z)) * w
-//   head_gate            out[t, h, :] = o[h, t, :] * sigmoid(gate[t, h])
+//   head_gate            out[t, h, :] = o[h, t, :] * sigmoid(gate[t, h]), or
+//                        entry by entry with a gate of H*dv columns
 //   xielu                piecewise quadratic / exponential activation
 //   softcap_             logits <- cap * tanh(logits / cap)
 #include "elem.h"
@@ -123,17 +124,19 @@ void gated_group_rmsnorm(torch::Tensor out, torch::Tensor y, torch::Tensor z,
   HIP_CHECK_KERNEL();
 }
 
+// gw: gate columns per head (1: one gate per head, dv: one per entry)
 template <typename T>
 __global__ __launch_bounds__(256) void head_gate_kernel(
     T* __restrict__ out, const T* __restrict__ o, const T* __restrict__ gate,
-    long ldg, long rows, int H, int dv) {
+    long ldg, long rows, int H, int dv, int gw) {
   const long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
   const long total = rows * H * dv;
   if (i >= total) return;
   const int d = (int)(i % dv);
   const int h = (int)((i / dv) % H);
   const long t = i / ((long)dv * H);
-  const float g = 1.0f / (1.0f + __expf(-ldf(gate + t * ldg + h)));
+  const long gc = gw == 1 ? h : (long)h * dv + d;
+  const float g = 1.0f / (1.0f + __expf(-ldf(gate + t * ldg + gc)));
   stf(out + i, ldf(o + ((long)h * rows + t) * dv + d) * g);
 }
 
@@ -141,42 +144,53 @@ __global__ __launch_bounds__(256) void head_gate_kernel(
 template <typename T>
 __global__ __launch_bounds__(256) void head_gate_vec_kernel(
     T* __restrict__ out, const T* __restrict__ o, const T* __restrict__ gate,
-    long ldg, long rows, int H, int dv) {
+    long ldg, long rows, int H, int dv, int gw) {
   const long i = ((long)blockIdx.x * blockDim.x + threadIdx.x) * 8;
   const long total = rows * H * dv;
   if (i >= total) return;
   const int d = (int)(i % dv);
   const int h = (int)((i / dv) % H);
   const long t = i / ((long)dv * H);
-  const float g = 1.0f / (1.0f + __expf(-ldf(gate + t * ldg + h)));
   float v[8];
   ld8(o + ((long)h * rows + t) * dv + d, v);
+  if (gw == 1) {
+    const float g = 1.0f / (1.0f + __expf(-ldf(gate + t * ldg + h)));
 #pragma unroll
-  for (int k = 0; k < 8; ++k) v[k] *= g;
+    for (int k = 0; k < 8; ++k) v[k] *= g;
+  } else {
+    float g[8];
+    ld8(gate + t * ldg + (long)h * dv + d, g);
+#pragma unroll
+    for (int k = 0; k < 8; ++k) v[k] *= 1.0f / (1.0f + expf(-g[k]));
+  }
   st8(out + i, v);
 }
 
-// out [T, H*dv]; o [H, T, dv] contiguous; gate [T, H] (any row stride).
+// out [T, H*dv]; o [H, T, dv] contiguous; gate [T, H] or [T, H*dv] (any row
+// stride).
 void head_gate(torch::Tensor out, torch::Tensor o, torch::Tensor gate) {
   check_act(out, "out"); check_act(o, "o"); check_act(gate, "gate");
   TORCH_CHECK(o.dim() == 3 && o.is_contiguous() && out.is_contiguous());
   const long H = o.size(0), rows = o.size(1), dv = o.size(2);
   TORCH_CHECK(out.dim() == 2 && out.size(0) == rows && out.size(1) == H * dv);
-  TORCH_CHECK(gate.dim() == 2 && gate.size(0) == rows && gate.size(1) == H &&
+  TORCH_CHECK(gate.dim() == 2 && gate.size(0) == rows &&
+              (gate.size(1) == H || gate.size(1) == H * dv) &&
               gate.stride(1) == 1);
+  const int gw = gate.size(1) == H ? 1 : (int)dv;
   TORCH_CHECK(o.scalar_type() == out.scalar_type() &&
               gate.scalar_type() == out.scalar_type());
   const long total = rows * H * dv;
   if (total == 0) return;
   auto stream = c10::hip::getCurrentHIPStream().stream();
-  if (dv % 8 == 0 && aligned16(out.data_ptr()) && aligned16(o.data_ptr())) {
+  if (dv % 8 == 0 && aligned16(out.data_ptr()) && aligned16(o.data_ptr()) &&
+      (gw == 1 || (gate.stride(0) % 8 == 0 && aligned16(gate.data_ptr())))) {
     KK_DISPATCH_ACT(out, {
       head_gate_vec_kernel<T><<<dim3((unsigned)((total / 8 + 255) / 256)), 256,
                                 0, stream>>>(
           reinterpret_cast<T*>(out.data_ptr()),
           reinterpret_cast<const T*>(o.data_ptr()),
           reinterpret_cast<const T*>(gate.data_ptr()), (long)gate.stride(0),
-          rows, (int)H, (int)dv);
+          rows, (int)H, (int)dv, gw);
     });
     HIP_CHECK_KERNEL();
     return;
@@ -187,7 +201,7 @@ void head_gate(torch::Tensor out, torch::Tensor o, torch::Tensor gate) {
         reinterpret_cast<T*>(out.data_ptr()),
         reinterpret_cast<const T*>(o.data_ptr()),
         reinterpret_cast<const T*>(gate.data_ptr()), (long)gate.stride(0),
-        rows, (int)H, (int)dv);
+        rows, (int)H, (int)dv, gw);
   });
   HIP_CHECK_KERNEL();
 }

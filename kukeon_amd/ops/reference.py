@@ -544,10 +544,12 @@ def latent_attention(out, q_abs, q, cache, cs, positions, row_seq,
 
 
 def head_gate(out, o, gate) -> None:
-    """out[t, h*dv:(h+1)*dv] = o[h, t] * sigmoid(gate[t, h])."""
+    """out[t, h*dv:(h+1)*dv] = o[h, t] * sigmoid(gate[t, h]); a gate with
+    H*dv columns acts entry by entry."""
     Hh, T, dv = o.shape
-    g = torch.sigmoid(gate.float())                          # [T, H]
-    out.copy_((o.float().permute(1, 0, 2) * g[:, :, None]).reshape(
+    g = torch.sigmoid(gate.float())                  # [T, H] or [T, H*dv]
+    g = g.view(T, Hh, -1)                            # per head or per entry
+    out.copy_((o.float().permute(1, 0, 2) * g).reshape(
         T, Hh * dv).to(out.dtype))
 
 
@@ -587,3 +589,141 @@ def relu_square_(x) -> None:
 def combine_rows(out, inp, inv) -> None:
     """out[t] = mean over k of inp[inv[t, k]]."""
     out.copy_(inp[inv.long()].float().mean(1).to(out.dtype))
+
+
+# ---------------------------------------------------------------------------
+# hybrid group (output-side layer norm, chunk-masked attention with a score
+# cap, linear attention with a fixed per-head decay, routed experts)
+# ---------------------------------------------------------------------------
+
+def _layer_norm(v: torch.Tensor, w: torch.Tensor, eps: float) -> torch.Tensor:
+    d = v - v.mean(-1, keepdim=True)
+    return d / torch.sqrt(d.pow(2).mean(-1, keepdim=True) + eps) * w
+
+
+def layernorm_residual(x, y, w, eps: float, out) -> None:
+    """x (fp32, in place) += layernorm(y) * w; out = x in the activation
+    format (the next sublayer reads the stream itself)."""
+    x += _layer_norm(y.float(), w, eps)
+    out.copy_(x.to(out.dtype))
+
+
+def layernorm(out, x, w, eps: float) -> None:
+    out.copy_(_layer_norm(x.float(), w, eps).to(out.dtype))
+
+
+def gelu_glu(out, gate, up) -> None:
+    """out = gelu_tanh(gate) * up."""
+    g = gate.float()
+    a = 0.5 * g * (1.0 + torch.tanh(0.7978845608028654 *
+                                    (g + 0.044715 * g * g * g)))
+    out.copy_((a * up.float()).to(out.dtype))
+
+
+def qk_norm_append(q_out, k_cache, v_cache, proj, q_col: int, k_col: int,
+                   v_col: int, wq, wk, eps: float, positions, row_seq,
+                   block_table) -> None:
+    """q_out = rmsnorm(proj[:, q_col:+Cq]) * wq over the whole projection
+    row; with caches given, the token's page rows get rmsnorm(k) * wk and
+    v. k_cache [blocks, G, BS, d], v_cache [blocks, G, BS, dv]."""
+    Cq = wq.numel()
+    own = k_cache is not None and k_cache.numel() > 0
+    for r in range(proj.shape[0]):
+        p = int(positions[r])
+        if p < 0:
+            continue
+        row = proj[r].float()
+        q_out[r] = (_unit_rms(row[q_col: q_col + Cq], eps) * wq).to(
+            q_out.dtype)
+        if not own:
+            continue
+        G, BS, d = k_cache.shape[1], k_cache.shape[2], k_cache.shape[3]
+        dv = v_cache.shape[3]
+        k = _unit_rms(row[k_col: k_col + G * d], eps) * wk
+        v = row[v_col: v_col + G * dv]
+        blk = int(block_table[int(row_seq[r]), p // BS])
+        k_cache[blk, :, p % BS] = k.view(G, d).to(k_cache.dtype)
+        v_cache[blk, :, p % BS] = v.view(G, dv).to(v_cache.dtype)
+
+
+def chunk_attention(out, q, k_cache, v_cache, positions, row_seq,
+                    block_table, H: int, scale: float, softcap: float,
+                    chunk: int) -> None:
+    """Grouped-query attention of row r (position p) over the keys
+    lo .. p with lo = the first position of p's chunk (0 without chunks);
+    scores are capped as softcap tanh(score / softcap) when softcap > 0."""
+    G, BS = k_cache.shape[1], k_cache.shape[2]
+    d, dv = k_cache.shape[3], v_cache.shape[3]
+    for r in range(q.shape[0]):
+        p = int(positions[r])
+        if p < 0:
+            out[r] = 0
+            continue
+        s = int(row_seq[r])
+        lo = (p // chunk) * chunk if chunk > 0 else 0
+        js = torch.arange(lo, p + 1)
+        blk = block_table[s, (js // BS).long()].long()
+        k = k_cache[blk, :, (js % BS).long()].float()         # [n, G, d]
+        v = v_cache[blk, :, (js % BS).long()].float()
+        qr = q[r].float().view(H, d)
+        for h in range(H):
+            g = h // (H // G)
+            sc = (k[:, g] @ qr[h]) * scale
+            if softcap > 0:
+                sc = softcap * torch.tanh(sc / softcap)
+            out[r, h * dv:(h + 1) * dv] = (torch.softmax(sc, -1) @
+                                           v[:, g]).to(out.dtype)
+
+
+def lightning_scan(y, proj, q_col: int, k_col: int, v_col: int, decay, state,
+                   positions, cu_rows, state_slots, H: int, d: int,
+                   dv: int) -> None:
+    """Linear attention with a fixed decay per head, token after token:
+    q, k, v = silu of the projection columns; S = decay_h S + k v^T;
+    y = S^T q. state [slots, H, dv, d] fp32 holds S^T (taken as zeros at
+    position 0); y [T, H*dv] fp32."""
+    nseq = cu_rows.numel() - 1
+    silu = lambda z: z * torch.sigmoid(z)
+    for s in range(nseq):
+        r0, r1 = int(cu_rows[s]), int(cu_rows[s + 1])
+        if r1 <= r0:
+            continue
+        if int(positions[r0]) < 0:
+            y[r0:r1] = 0
+            continue
+        slot = int(state_slots[s])
+        S = state[slot].transpose(1, 2).clone()              # [H, d, dv]
+        if int(positions[r0]) == 0:
+            S.zero_()
+        for r in range(r0, r1):
+            row = proj[r].float()
+            qq = silu(row[q_col: q_col + H * d]).view(H, d)
+            kk = silu(row[k_col: k_col + H * d]).view(H, d)
+            vv = silu(row[v_col: v_col + H * dv]).view(H, dv)
+            S = decay[:, None, None] * S + kk[:, :, None] * vv[:, None, :]
+            y[r] = (S * qq[:, :, None]).sum(1).reshape(H * dv)
+        state[slot] = S.transpose(1, 2)
+
+
+def gated_rmsnorm(out, y, gate, w, eps: float) -> None:
+    """out = rmsnorm(y) * w * sigmoid(gate), the norm over the whole row."""
+    out.copy_((_unit_rms(y.float(), eps) * w *
+               torch.sigmoid(gate.float())).to(out.dtype))
+
+
+def router_topk(idx, wts, logits, top: int, dense_rows: int = 0) -> None:
+    """The `top` largest logits of every row (ties: the lower index) and the
+    softmax over just those. With dense_rows = T the index written is
+    expert * T + row: the row of that pair in an [E, T, W] result."""
+    val, ix = torch.sort(logits.float(), dim=-1, descending=True, stable=True)
+    val, ix = val[:, :top], ix[:, :top]
+    wts.copy_(torch.softmax(val, -1))
+    if dense_rows:
+        ix = ix * dense_rows + torch.arange(logits.shape[0])[:, None]
+    idx.copy_(ix.to(idx.dtype))
+
+
+def combine_rows_weighted(out, inp, inv, wts) -> None:
+    """out[t] = sum over k of wts[t, k] * inp[inv[t, k]]."""
+    out.copy_((inp[inv.long()].float() * wts[:, :, None]).sum(1).to(
+        out.dtype))
