@@ -30,18 +30,23 @@ COMPARE_SIZES = {
 
 
 def compare_families(args) -> None:
-    """Prefill and decode tokens/s of Lipedra or Rasesun and of Llama
-    through the same engine at equal sizes: same width, head counts,
+    """Prefill and decode tokens/s of Lipedra, Rasesun or Dumovik and of
+    Llama (or another family) through the same engine at equal sizes: same
+    width, head counts,
     feed-forward size, layer count and vocabulary (Llama head_dim 128;
     Lipedra two score maps of 64 and value rows of 128 — equal cache bytes
     per token; Rasesun three state-space layers to one latent-attention
     layer with a 1024-token window, every second feed-forward a mixture of
-    16 table-routed experts, two active)."""
+    16 table-routed experts, two active; Dumovik periods of chunk-local
+    attention over 512-token chunks, two linear-attention layers and latent
+    attention, every second feed-forward a mixture of 16 routed experts, two
+    active)."""
     from kukeon_amd.engine.config import (EngineConfig, ModelConfig,
                                           SamplingParams)
     from kukeon_amd.engine.engine import LLMEngine
     from kukeon_amd.engine.kv_cache import SequenceKV
     from kukeon_amd.models import registry
+    from kukeon_amd.models.dumovik import dumovik_bench
     from kukeon_amd.models.lipedra import lipedra_bench
     from kukeon_amd.models.rasesun import rasesun_bench
 
@@ -54,7 +59,7 @@ def compare_families(args) -> None:
         W, hq, hk, ff, nl = COMPARE_SIZES[size]
         if not on_gpu:
             W, hq, hk, ff, nl = 256, 2, 2, 512, 2
-        for fam in ("llama", args.compare_family):
+        for fam in (args.compare_against, args.compare_family):
             if fam == "llama":
                 cfg = ModelConfig(name=f"llama-{size}", hidden_size=W,
                                   num_layers=nl, num_q_heads=hq,
@@ -67,6 +72,12 @@ def compare_families(args) -> None:
                                     window=1024 if on_gpu else 16,
                                     experts=16 if on_gpu else 4,
                                     name=f"rasesun-{size}")
+            elif fam == "dumovik":
+                cfg = dumovik_bench(width=W, layers=nl, heads=hq,
+                                    kv_heads=hk, ff=ff, vocab=vocab,
+                                    chunk=512 if on_gpu else 16,
+                                    experts=16 if on_gpu else 4,
+                                    name=f"dumovik-{size}")
             else:
                 cfg = lipedra_bench(width=W, layers=nl, heads=hq,
                                     kv_heads=hk, dim=64, vdim=128, ff=ff,
@@ -150,9 +161,13 @@ def main() -> None:
                          "decode throughput of the Lipedra family beside "
                          "Llama at equal layer sizes (random weights)")
     ap.add_argument("--compare-family", default="lipedra",
-                    choices=["lipedra", "rasesun"],
+                    choices=["lipedra", "rasesun", "dumovik"],
                     help="with --compare-families: the family that runs "
                          "beside Llama")
+    ap.add_argument("--compare-against", default="llama",
+                    choices=["llama", "lipedra", "rasesun"],
+                    help="with --compare-families: the family it runs "
+                         "beside (default Llama)")
     ap.add_argument("--compare-sizes", default="2k,4k,8k",
                     help="with --compare-families: which of 2k,4k,8k")
     args = ap.parse_args()

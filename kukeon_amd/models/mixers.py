@@ -368,9 +368,18 @@ class ChunkedAttention(nn.Module):
                            self.k_norm, self.eps, meta.positions,
                            meta.row_seq, meta.block_table)
         o = torch.empty(T, m.heads * m.vdim, dtype=h.dtype, device=h.device)
-        ops.chunk_attention(o, q, cache, cache_v, meta.positions,
-                            meta.row_seq, meta.block_table, m.heads, m.scale,
-                            m.softcap, m.chunk)
+        if (meta.mode == "prefill" and meta.max_rows >= 16 and
+                meta.qb_seq is not None and
+                ops.chunk_tiles_supported(q, m.dim, m.vdim, cache.shape[2])):
+            # prompt portions on the matrix cores
+            ops.chunk_attention_tiles(o, q, cache, cache_v, meta.block_table,
+                                      meta.seq_lens, meta.q_starts,
+                                      meta.qb_seq, meta.qb_start, m.scale,
+                                      m.softcap, m.chunk)
+        else:
+            ops.chunk_attention(o, q, cache, cache_v, meta.positions,
+                                meta.row_seq, meta.block_table, m.heads,
+                                m.scale, m.softcap, m.chunk)
         return ops.linear(o, self.w_o)
 
 

@@ -639,6 +639,21 @@ def chunk_attention(out, q, k_cache, v_cache, positions, row_seq,
                             block_table, H, scale, softcap, chunk)
 
 
+def chunk_tiles_supported(t: torch.Tensor, d: int, dv: int, BS: int) -> bool:
+    """Whether the matrix-core kernel for prompt portions serves these
+    sizes (bf16 on a GPU only)."""
+    return (t.is_cuda and t.dtype == torch.bfloat16
+            and _hyb(t).chunk_attention_tiles_supported(d, dv, BS))
+
+
+def chunk_attention_tiles(out, q, k_cache, v_cache, block_table, seq_lens,
+                          q_starts, qb_seq, qb_start, scale: float,
+                          softcap: float, chunk: int) -> None:
+    _hyb(q).chunk_attention_tiles(out, q, k_cache, v_cache, block_table,
+                                  seq_lens, q_starts, qb_seq, qb_start,
+                                  scale, softcap, chunk)
+
+
 def lightning_scan(y, proj, q_col: int, k_col: int, v_col: int, decay, state,
                    positions, cu_rows, state_slots, H: int, d: int,
                    dv: int) -> None:

@@ -55,6 +55,7 @@ HYB_SOURCES = [
     "layer_norm.hip",
     "glu_clamp.hip",
     "chunk_attn.hip",
+    "prefill_attn.hip",
     "lightning.hip",
     "routed_moe.hip",
     "latent_attn.hip",

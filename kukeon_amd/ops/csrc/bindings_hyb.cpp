@@ -24,6 +24,13 @@ void chunk_attention(torch::Tensor out, torch::Tensor q, torch::Tensor k_cache,
                      torch::Tensor v_cache, torch::Tensor positions,
                      torch::Tensor row_seq, torch::Tensor block_table,
                      int64_t H, double scale, double softcap, int64_t chunk);
+bool chunk_attention_tiles_supported(int64_t d, int64_t dv, int64_t BS);
+void chunk_attention_tiles(torch::Tensor out, torch::Tensor q,
+                           torch::Tensor k_cache, torch::Tensor v_cache,
+                           torch::Tensor block_table, torch::Tensor seq_lens,
+                           torch::Tensor q_starts, torch::Tensor qb_seq,
+                           torch::Tensor qb_start, double scale,
+                           double softcap, int64_t chunk);
 void lightning_scan(torch::Tensor y, torch::Tensor proj, int64_t q_col,
                     int64_t k_col, int64_t v_col, torch::Tensor decay,
                     torch::Tensor state, torch::Tensor positions,
@@ -60,6 +67,10 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
         "whole-projection q/k norms, paged K/V append");
   m.def("chunk_attention", &kukeon::chunk_attention,
         "grouped-query attention over the query's own chunk, capped scores");
+  m.def("chunk_attention_tiles_supported",
+        &kukeon::chunk_attention_tiles_supported);
+  m.def("chunk_attention_tiles", &kukeon::chunk_attention_tiles,
+        "chunk-local attention for prompt portions on the matrix cores");
   m.def("lightning_scan", &kukeon::lightning_scan,
         "linear attention with a fixed decay per head, carried fp32 state");
   m.def("gated_rmsnorm", &kukeon::gated_rmsnorm,

@@ -1,4 +1,5 @@
-// Varlen causal paged prefill attention (MFMA, bf16) for gfx950 — plus the
+// Varlen causal paged prefill attention (MFMA, bf16) for gfx950, also in a
+// chunk-local form with capped scores (template flag EXT) — plus the
 // fragment-layout probe used by the GPU test suite to pin the
 // v_mfma_f32_32x32x16_bf16 operand maps this kernel relies on.
 //
@@ -122,7 +123,11 @@ DEV_INLINE unsigned int cvt_pk_bf16(float lo, float hi) {
 
 // ---------- the kernel ----------
 // D=128, QBLK=32 rows per workgroup, KV tile = 32 tokens (2 cache blocks).
-template <int BS, bool FP8>
+// EXT adds what chunk-local attention with capped scores needs: keys start at
+// the first position of the query's chunk, scores pass cap * tanh(s / cap),
+// and the softmax weights enter the PV product as hi + lo (two bf16 terms)
+// so that they keep fp32-grade accuracy.
+template <int BS, bool FP8, bool EXT>
 __global__ __launch_bounds__(256, 1) void prefill_attn_kernel(
     unsigned short* __restrict__ out,       // [T, Hq*D]
     const unsigned short* __restrict__ q,   // [T, q_stride] fused qkv rows
@@ -134,7 +139,7 @@ __global__ __launch_bounds__(256, 1) void prefill_attn_kernel(
     const int* __restrict__ qb_seq,         // [nqb]
     const int* __restrict__ qb_start,       // [nqb] local q offset
     long q_stride, long q_offset, int Hq, int Hk, int max_blocks,
-    int out_stride, float scale) {
+    int out_stride, float scale, float cap, int chunk) {
   constexpr int D = 128;
   constexpr int KVT = 32;
   // 16-B aligned: staged via uint4 stores (guide G17)
@@ -161,6 +166,10 @@ __global__ __launch_bounds__(256, 1) void prefill_attn_kernel(
 
   // absolute position of this lane's q column (clamped for padding rows)
   const int q_abs = abs_start + qb0 + min(qcol, qn - 1);
+  // first key this lane's query sees, and the first any row of the tile sees
+  const int q_lo = (EXT && chunk > 0) ? (q_abs / chunk) * chunk : 0;
+  const int tile_lo =
+      (EXT && chunk > 0) ? ((abs_start + qb0) / chunk) * chunk : 0;
 
   // ---- load Q fragments (B-operand: col=q, k=d chunks) ----
   unsigned int qfrag[8][4];
@@ -182,7 +191,7 @@ __global__ __launch_bounds__(256, 1) void prefill_attn_kernel(
   const int ntiles = (kv_limit + KVT - 1) / KVT;
   const int nblocks = (ctx + BS - 1) / BS;
 
-  for (int ti = 0; ti < ntiles; ++ti) {
+  for (int ti = tile_lo / KVT; ti < ntiles; ++ti) {
     const int kvbase = ti * KVT;
     // ---- cooperative stage ----
     {
@@ -278,8 +287,11 @@ __global__ __launch_bounds__(256, 1) void prefill_attn_kernel(
     for (int r = 0; r < 16; ++r) {
       const int kvrow = (r & 3) + 8 * (r >> 2) + 4 * hi;
       const int kvpos = kvbase + kvrow;
-      const bool valid = (kvpos <= q_abs) && (kvpos < ctx);
-      sv[r] = valid ? sacc[r] * scale : -INFINITY;
+      const bool valid = (kvpos <= q_abs) && (kvpos < ctx) &&
+                         (!EXT || kvpos >= q_lo);
+      float sc = sacc[r] * scale;
+      if (EXT && cap > 0.f) sc = cap * tanhf(sc / cap);
+      sv[r] = valid ? sc : -INFINITY;
       tmax = fmaxf(tmax, sv[r]);
     }
     tmax = fmaxf(tmax, __shfl_xor(tmax, 32, WAVE));
@@ -315,6 +327,27 @@ __global__ __launch_bounds__(256, 1) void prefill_attn_kernel(
       pb[c][0] = s1[0]; pb[c][1] = s2[0];
       pb[c][2] = s1[1]; pb[c][3] = s2[1];
     }
+    // what the rounding to bf16 dropped, as a second set of fragments
+    unsigned int pl[2][4];
+    if (EXT) {
+      unsigned int cl[8];
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        const float h0 = us2f((unsigned short)(cp[j] & 0xffffu));
+        const float h1 = us2f((unsigned short)(cp[j] >> 16));
+        cl[j] = cvt_pk_bf16(p[2 * j] - h0, p[2 * j + 1] - h1);
+      }
+#pragma unroll
+      for (int c = 0; c < 2; ++c) {
+        const int b0 = 4 * c;
+        auto s1 = __builtin_amdgcn_permlane32_swap(cl[b0 + 0], cl[b0 + 2],
+                                                   false, false);
+        auto s2 = __builtin_amdgcn_permlane32_swap(cl[b0 + 1], cl[b0 + 3],
+                                                   false, false);
+        pl[c][0] = s1[0]; pl[c][1] = s2[0];
+        pl[c][2] = s1[1]; pl[c][3] = s2[1];
+      }
+    }
 
     // ---- O^T += V^T · P^T ----
 #pragma unroll
@@ -329,6 +362,11 @@ __global__ __launch_bounds__(256, 1) void prefill_attn_kernel(
             as_frag(vf.x, vf.y, vf.z, vf.w),
             as_frag(pb[c][0], pb[c][1], pb[c][2], pb[c][3]),
             oacc[db], 0, 0, 0);
+        if (EXT)
+          oacc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
+              as_frag(vf.x, vf.y, vf.z, vf.w),
+              as_frag(pl[c][0], pl[c][1], pl[c][2], pl[c][3]),
+              oacc[db], 0, 0, 0);
       }
     }
   }
@@ -372,16 +410,67 @@ void prefill_attention(torch::Tensor out, torch::Tensor q,
   dim3 grid(nqb, Hk, (G + 3) / 4);
   const bool fp8 = k_cache.scalar_type() == torch::kUInt8;
 #define PF_LAUNCH(FP8_)                                                      \
-  prefill_attn_kernel<16, FP8_><<<grid, 256, 0, stream>>>(                   \
+  prefill_attn_kernel<16, FP8_, false><<<grid, 256, 0, stream>>>(            \
       reinterpret_cast<unsigned short*>(out.data_ptr()),                     \
       reinterpret_cast<const unsigned short*>(q.data_ptr()),                 \
       k_cache.data_ptr(), v_cache.data_ptr(), block_table.data_ptr<int>(),   \
       seq_lens.data_ptr<int>(), q_starts.data_ptr<int>(),                    \
       qb_seq.data_ptr<int>(), qb_start.data_ptr<int>(), q.stride(0),         \
       q_offset, Hq, Hk, (int)block_table.size(1), (int)out.stride(0),        \
-      (float)scale)
+      (float)scale, 0.f, 0)
   if (fp8) { PF_LAUNCH(true); } else { PF_LAUNCH(false); }
 #undef PF_LAUNCH
+  HIP_CHECK_KERNEL();
+}
+
+// sizes the tile kernel serves for chunk-local attention
+bool chunk_attention_tiles_supported(int64_t d, int64_t dv, int64_t BS) {
+  return d == 128 && dv == 128 && BS == 16;
+}
+
+// Prompt portions of chunk-local attention on the matrix cores (bf16, heads
+// of 128, pages of 16): out [T, H*128], q [T, H*128] contiguous, caches
+// [blocks, G, 16, 128]; the row maps are the ones of prefill_attention.
+void chunk_attention_tiles(torch::Tensor out, torch::Tensor q,
+                           torch::Tensor k_cache, torch::Tensor v_cache,
+                           torch::Tensor block_table, torch::Tensor seq_lens,
+                           torch::Tensor q_starts, torch::Tensor qb_seq,
+                           torch::Tensor qb_start, double scale,
+                           double softcap, int64_t chunk) {
+  TORCH_CHECK(k_cache.dim() == 4 && v_cache.dim() == 4 &&
+              k_cache.is_contiguous() && v_cache.is_contiguous());
+  const int Hk = (int)k_cache.size(1);
+  TORCH_CHECK(chunk_attention_tiles_supported(k_cache.size(3),
+                                              v_cache.size(3),
+                                              k_cache.size(2)));
+  TORCH_CHECK(q.scalar_type() == torch::kBFloat16 &&
+              out.scalar_type() == torch::kBFloat16 &&
+              k_cache.scalar_type() == torch::kBFloat16 &&
+              v_cache.scalar_type() == torch::kBFloat16);
+  TORCH_CHECK(q.dim() == 2 && q.is_contiguous() && out.dim() == 2 &&
+              out.is_contiguous() && out.size(0) == q.size(0) &&
+              out.size(1) == q.size(1) && q.size(1) % 128 == 0);
+  const int Hq = (int)(q.size(1) / 128);
+  TORCH_CHECK(Hq % Hk == 0 && chunk >= 0);
+  TORCH_CHECK(q_starts.dim() == 2 && q_starts.size(1) == 2);
+  TORCH_CHECK(qb_seq.scalar_type() == torch::kInt32 &&
+              qb_start.scalar_type() == torch::kInt32 &&
+              seq_lens.scalar_type() == torch::kInt32 &&
+              block_table.scalar_type() == torch::kInt32 &&
+              q_starts.scalar_type() == torch::kInt32);
+  const int nqb = (int)qb_seq.size(0);
+  if (nqb == 0) return;
+  const int G = Hq / Hk;
+  auto stream = c10::hip::getCurrentHIPStream().stream();
+  dim3 grid(nqb, Hk, (G + 3) / 4);
+  prefill_attn_kernel<16, false, true><<<grid, 256, 0, stream>>>(
+      reinterpret_cast<unsigned short*>(out.data_ptr()),
+      reinterpret_cast<const unsigned short*>(q.data_ptr()),
+      k_cache.data_ptr(), v_cache.data_ptr(), block_table.data_ptr<int>(),
+      seq_lens.data_ptr<int>(), q_starts.data_ptr<int>(),
+      qb_seq.data_ptr<int>(), qb_start.data_ptr<int>(), q.stride(0), 0L, Hq,
+      Hk, (int)block_table.size(1), (int)out.stride(0), (float)scale,
+      (float)softcap, (int)chunk);
   HIP_CHECK_KERNEL();
 }
 

@@ -102,6 +102,16 @@ CONFIGS = {
         layer(attn(heads=2, kv_heads=1, dim=8, vdim=8, chunk=300), None),
         layer(latent(heads=1, dim=8, rot_dim=2, vdim=3, kv_rank=16), None),
     ], width=16, vocab=21),
+    # heads of 128 on pages of 16: the sizes of the matrix-core attention
+    # kernel that long portions take; chunks that end inside a key tile, a
+    # sharing layer without chunks or cap, three query heads per kv head
+    "tiles": lambda: config([
+        layer(attn(heads=6, kv_heads=2, dim=128, vdim=128, chunk=40,
+                   softcap=6.0, scale=0.3), dense(48)),
+        layer(lightning(heads=2, dim=8, vdim=8), None),
+        layer(attn(heads=6, kv_heads=2, dim=128, vdim=128, chunk=0,
+                   softcap=0, scale=0.2, kv_from=0), None),
+    ], width=48, vocab=40),
     # a chunk longer than one pass of the attention kernel over the keys
     "long_chunk": lambda: config([
         layer(attn(heads=2, kv_heads=1, dim=8, vdim=8, chunk=150,
@@ -205,23 +215,35 @@ def make_engine(cfg, tensors, device, dtype, blocks=96, slots=4,
 
 
 def tol(dtype):
-    return 2e-4 if dtype == "fp32" else 0.12
+    return 2e-4 if dtype == "fp32" else 0.08
 
 
-def rel_err(got, want):
-    """Error of logits rows as the ratio of centred root mean squares."""
+def row_errors(got, want):
+    """Error of every logits row as the ratio of centred root mean
+    squares."""
     got = got.detach().cpu().double()
     want = want.detach().cpu().double()
     d = got - want
     d = d - d.mean(-1, keepdim=True)
     w = want - want.mean(-1, keepdim=True)
-    return float((d.pow(2).mean(-1).sqrt() /
-                  w.pow(2).mean(-1).sqrt().clamp_min(1e-9)).max())
+    return (d.pow(2).mean(-1).sqrt() /
+            w.pow(2).mean(-1).sqrt().clamp_min(1e-9)).reshape(-1)
 
 
 def check(got, want, dtype, what=""):
-    e = rel_err(got, want)
-    assert e <= tol(dtype), f"{what}: error {e:.3g} over {tol(dtype)}"
+    """fp32: every row within the tolerance. bf16: rounding can flip a close
+    call of a router for a single token, which moves that row by much more
+    than rounding does elsewhere, so one row in ten (at least one) may be
+    off, though never as far as a wrong mechanism puts it."""
+    e = row_errors(got, want)
+    if dtype == "fp32":
+        assert float(e.max()) <= tol(dtype), \
+            f"{what}: error {float(e.max()):.3g} over {tol(dtype)}"
+        return
+    allowed = max(1, e.numel() // 10)
+    over = int((e > tol(dtype)).sum())
+    assert over <= allowed and float(e.max()) <= 0.5, \
+        f"{what}: {over} rows over {tol(dtype)}, worst {float(e.max()):.3g}"
 
 
 def logits_of(cfg, W, toks):
@@ -393,6 +415,26 @@ def case_long_chunk(device, dtype):
     check(got, want, dtype, "portions and decoding")
 
 
+def case_long_portions(device, dtype):
+    """Portions long enough for the matrix-core attention kernel beside
+    short ones and single tokens that take the other form; cuts inside a
+    chunk and inside a key tile."""
+    cfg = CONFIGS["tiles"]()
+    W = weights(cfg, 13)
+    prompts = [tokens(cfg, n, 80 + n) for n in (300, 70)]
+    want = [logits_of(cfg, W, p) for p in prompts]
+    eng = make_engine(cfg, W, device, dtype, blocks=30, block_size=16,
+                      max_len=400)
+    got = run_schedule(eng, prompts, [[(0, 300), (1, 69)], [(1, 1)]])
+    for i in range(2):
+        check(got[i], want[i], dtype, f"whole, request {i}")
+    got = run_schedule(eng, prompts,
+                       [[(0, 21)], [(0, 270), (1, 2)], [(0, 1), (1, 68)],
+                        [(0, 8)]])
+    for i in range(2):
+        check(got[i], want[i], dtype, f"portions, request {i}")
+
+
 def case_sorted_experts(device, dtype):
     """Long portions sort their rows by expert and run each expert over its
     rows at once; short steps run every expert on every row. Both against
@@ -549,3 +591,271 @@ def case_router(device, dtype):
         eng = make_engine(cfg, W, device, dtype)
         got = run_schedule(eng, [toks], [[(0, 70)], [(0, 9)], [(0, 1)]])[0]
         check(got, want, dtype, f"top {top}")
+
+
+# ------------------------------------------------ the framework's entry points
+def assert_greedy(cfg, W, prompt, got, what=""):
+    """Every generated token is the plain model's best one, up to the
+    rounding of the logits to bfloat16 that the sampler works on."""
+    toks = list(prompt)
+    for i, t in enumerate(got):
+        lg = logits_of(cfg, W, toks)[-1]
+        best = float(lg.max())
+        assert float(lg[t]) >= best - abs(best) * 2.0 ** -7, \
+            f"{what}: token {i} is {t}, the plain model says " \
+            f"{int(lg.argmax())}"
+        toks.append(t)
+
+
+def _generate(eng, kv, prompt, n):
+    sp = SamplingParams(temperature=0.0, max_new_tokens=n)
+    eng.add_request(kv, prompt, sp)
+    out = []
+    while eng.has_work():
+        for o in eng.step():
+            out.extend(o.new_tokens)
+    return out
+
+
+def case_multi_turn(device, dtype):
+    """A session's second turn continues from its pages and state slot; an
+    idle session whose pages and slot were taken away is rebuilt from its
+    history."""
+    cfg = CONFIGS["hybrid"]()
+    W = weights(cfg, 15)
+    eng = make_engine(cfg, W, device, dtype, blocks=12, slots=2, max_len=64,
+                      poison=False, decode_microbatch=2)
+    a, b = SequenceKV(4), SequenceKV(4)
+    p1, p2, p3 = tokens(cfg, 9, 60), tokens(cfg, 5, 61), tokens(cfg, 30, 62)
+    t1 = _generate(eng, a, p1, 4)
+    assert_greedy(cfg, W, p1, t1, "first turn")
+    t2 = _generate(eng, a, p2, 3)
+    assert_greedy(cfg, W, p1 + t1 + p2, t2, "second turn")
+    assert a.num_tokens > 0 and a.state_slot >= 0
+    tb = _generate(eng, b, p3, 4)       # needs a's pages
+    assert_greedy(cfg, W, p3, tb, "other session")
+    assert a.num_tokens == 0 and a.state_slot < 0 and a.history
+    eng.free_sequence(b)
+    t3 = _generate(eng, a, [7, 3], 3)
+    assert_greedy(cfg, W, p1 + t1 + p2 + t2 + [7, 3], t3, "rebuilt session")
+
+
+def write_checkpoint(folder, cfg, W):
+    """config.json and model.safetensors (8-byte header length, JSON header,
+    raw data) of a config dictionary and its tensors."""
+    import json
+    import os
+    import struct
+    with open(os.path.join(folder, "config.json"), "w") as f:
+        json.dump(cfg, f)
+    head, blobs, at = {}, [], 0
+    for name, t in W.items():
+        raw = t.view(torch.int16).contiguous().numpy().tobytes()
+        head[name] = {"dtype": "BF16", "shape": list(t.shape),
+                      "data_offsets": [at, at + len(raw)]}
+        blobs.append(raw)
+        at += len(raw)
+    hj = json.dumps(head).encode()
+    with open(os.path.join(folder, "model.safetensors"), "wb") as f:
+        f.write(struct.pack("<Q", len(hj)) + hj + b"".join(blobs))
+
+
+def case_registry(tmp_path, device, dtype):
+    """A checkpoint folder is found by its architecture name and read."""
+    from kukeon_amd.models.registry import load_checkpoint
+    cfg = CONFIGS["plain"]()
+    W = weights(cfg, 11)
+    write_checkpoint(tmp_path, cfg, W)
+    mcfg, model = load_checkpoint(str(tmp_path), device=device, dtype=dtype)
+    assert mcfg.family == "dumovik" and len(model.layers) == 3
+    eng = LLMEngine(model, mcfg, EngineConfig(
+        block_size=4, max_model_len=64, max_sessions=2, state_slots=2,
+        num_kv_blocks=16, use_graphs=False), device=device)
+    toks = tokens(cfg, 13, 11)
+    got = run_schedule(eng, [toks], [[(0, 6)], [(0, 7)]])[0]
+    check(got, logits_of(cfg, W, toks), dtype, "from a folder")
+
+
+def case_trace_runner(tmp_path, device, dtype):
+    """The trace runner as a program: a checkpoint folder, steps on standard
+    input, logits files and `done` lines back. Three requests through a pool
+    sized for two, portions beside single tokens, a request left out of a
+    step."""
+    import json
+    import os
+    import subprocess
+    import sys
+    import numpy as np
+    cfg = CONFIGS["hybrid"]()
+    W = weights(cfg, 14)
+    model_dir = tmp_path / "model"
+    out_dir = tmp_path / "out"
+    model_dir.mkdir()
+    write_checkpoint(model_dir, cfg, W)
+    prompts = {"a": tokens(cfg, 70, 90), "b": tokens(cfg, 40, 91),
+               "c": tokens(cfg, 33, 92)}
+    want = {k: logits_of(cfg, W, p) for k, p in prompts.items()}
+    steps = [[("a", 30), ("b", 1)], [("a", 1), ("b", 38)], [("a", 39)],
+             [("b", 1), ("c", 2)], [("c", 30)], [("c", 1)]]
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    cmd = [sys.executable, os.path.join(root, "bin", "trace_run"), "--model",
+           str(model_dir), "--dtype",
+           "float32" if dtype == "fp32" else "bfloat16", "--out",
+           str(out_dir), "--max-tokens", "128", "--slots", "2", "--device",
+           device]
+    p = subprocess.Popen(cmd, stdin=subprocess.PIPE, stdout=subprocess.PIPE,
+                         text=True, cwd=root)
+    at = {k: 0 for k in prompts}
+    try:
+        for n, step in enumerate(steps):
+            entries, end = [], []
+            for k, cnt in step:
+                toks = prompts[k][at[k]: at[k] + cnt]
+                entries.append({"id": k, "tokens": toks,
+                                "want": [0, cnt - 1] if cnt > 1 else [0]})
+                at[k] += cnt
+                if at[k] == len(prompts[k]):
+                    end.append(k)
+            p.stdin.write(json.dumps({"step": n, "entries": entries,
+                                      "end": end}) + "\n")
+            p.stdin.flush()
+            line = p.stdout.readline()
+            while line and line.strip() != "done %d" % n:
+                line = p.stdout.readline()
+            assert line, "the runner ended early"
+            got = np.fromfile(out_dir / ("%d.f32" % n), dtype="<f4").reshape(
+                -1, cfg["vocab"])
+            row = 0
+            for k, cnt in step:
+                a = at[k] - cnt
+                for w in ([0, cnt - 1] if cnt > 1 else [0]):
+                    check(torch.from_numpy(got[row].copy())[None],
+                          want[k][a + w][None], dtype, f"step {n} {k}+{w}")
+                    row += 1
+            assert row == got.shape[0]
+        p.stdin.close()
+        assert p.wait(timeout=60) == 0
+    finally:
+        if p.poll() is None:
+            p.kill()
+
+
+# ------------------------------------------------------- single operations
+def _act(dtype):
+    return torch.float32 if dtype == "fp32" else torch.bfloat16
+
+
+def _close(got, want, dtype, what):
+    got = got.detach().cpu().double()
+    want = want.detach().cpu().double()
+    e = float((got - want).abs().max()) / max(float(want.abs().max()), 1e-9)
+    lim = 2e-5 if dtype == "fp32" else 2e-2
+    assert e <= lim, f"{what}: error {e:.3g} over {lim}"
+
+
+def case_op_layer_norm(device, dtype):
+    """Output-side layer norm with the residual sum, and the plain one, for
+    rows on and off the vector path and wider than one pass."""
+    from kukeon_amd import ops
+    g = torch.Generator().manual_seed(31)
+    for T, Wd, ld in ((5, 40, 40), (3, 37, 50), (4, 2304, 2304),
+                      (2, 4104, 4200)):
+        x = torch.randn(T, Wd, generator=g)
+        y = (torch.randn(T, ld, generator=g) * 3 + 0.7).to(_act(dtype))
+        w = torch.randn(Wd, generator=g)
+        yd = y[:, :Wd].double()
+        want_x = x.double() + oracle.layer_norm(yd, w.double(), 1e-4)
+        xd = x.to(device).clone()
+        out = torch.empty(T, Wd, dtype=_act(dtype), device=device)
+        ops.layernorm_residual(xd, y.to(device)[:, :Wd], w.to(device), 1e-4,
+                               out)
+        _close(xd, want_x, "fp32", f"stream {Wd}")
+        _close(out, want_x, dtype, f"cast {Wd}")
+        ops.layernorm(out, xd, w.to(device), 1e-4)
+        _close(out, oracle.layer_norm(xd.cpu().double(), w.double(), 1e-4),
+               dtype, f"plain {Wd}")
+
+
+def case_op_gated(device, dtype):
+    """The gelu-gated product and the sigmoid-gated norm."""
+    from kukeon_amd import ops
+    g = torch.Generator().manual_seed(32)
+    for T, F in ((7, 24), (3, 13), (2, 4096 + 8)):
+        z = (torch.randn(T, 2 * F + 8, generator=g) * 2).to(_act(dtype))
+        zd = z.to(device)
+        out = torch.empty(T, F, dtype=_act(dtype), device=device)
+        ops.gelu_glu(out, zd[:, :F], zd[:, F + 8: 2 * F + 8])
+        want = oracle.gelu_tanh(z[:, :F].double()) * \
+            z[:, F + 8: 2 * F + 8].double()
+        _close(out, want, dtype, f"gelu {F}")
+        y = torch.randn(T, F, generator=g) * 4
+        w = torch.randn(F, generator=g)
+        ops.gated_rmsnorm(out, y.to(device), zd[:, :F], w.to(device), 1e-3)
+        want = oracle.unit_rms(y.double(), 1e-3) * w.double() * \
+            torch.sigmoid(z[:, :F].double())
+        _close(out, want, dtype, f"gated norm {F}")
+
+
+def case_op_scan(device, dtype, H=3, d=5, dv=7, cuts=(4, 1, 9, 1, 1)):
+    """The decayed recurrence over portions with a dirty slot and an
+    inactive neighbour, against the token-by-token sums."""
+    from kukeon_amd import ops
+    g = torch.Generator().manual_seed(33)
+    n = sum(cuts)
+    C = 2 * H * d + H * dv
+    proj = torch.randn(n, C + 3, generator=g).to(_act(dtype))
+    decay = torch.rand(H, generator=g) * 0.5 + 0.5
+    decay[-1] = 1.0
+    silu = lambda z: z * torch.sigmoid(z)
+    pd = proj.double()
+    q = silu(pd[:, 3: 3 + H * d]).view(n, H, d)
+    k = silu(pd[:, 3 + H * d: 3 + 2 * H * d]).view(n, H, d)
+    v = silu(pd[:, 3 + 2 * H * d:]).view(n, H, dv)
+    S = torch.zeros(H, d, dv, dtype=torch.float64)
+    want = torch.zeros(n, H * dv, dtype=torch.float64)
+    for i in range(n):
+        S = decay.double()[:, None, None] * S + \
+            k[i][:, :, None] * v[i][:, None, :]
+        want[i] = torch.einsum("hde,hd->he", S, q[i]).reshape(-1)
+    state = torch.full((3, H, dv, d), 9.0, device=device)
+    i32 = lambda x: torch.tensor(x, dtype=torch.int32, device=device)
+    got = []
+    at = 0
+    for c in cuts:
+        # a second, inactive sequence of one row rides along
+        rows = torch.cat([proj[at: at + c], proj[:1]]).to(device)
+        y = torch.full((c + 1, H * dv), 5.0, device=device)
+        ops.lightning_scan(y, rows, 3, 3 + H * d, 3 + 2 * H * d,
+                           decay.to(device), state,
+                           i32(list(range(at, at + c)) + [-1]),
+                           i32([0, c, c + 1]), i32([2, 0]), H, d, dv)
+        assert float(y[c].abs().max()) == 0.0
+        got.append(y[:c].cpu())
+        at += c
+    lim = "fp32" if dtype == "fp32" else "bf16"
+    _close(torch.cat(got), want, lim, f"scan {H}x{d}x{dv}")
+    assert float((state[0] - 9.0).abs().max()) == 0.0
+    _close(state[2].cpu().transpose(1, 2), S, "fp32", "carried state")
+
+
+def case_op_router(device, dtype):
+    """Top experts and their weights, ties and equal logits included."""
+    from kukeon_amd import ops
+    g = torch.Generator().manual_seed(34)
+    for T, E, top in ((9, 5, 2), (300, 12, 4), (4, 3, 3), (6, 7, 1)):
+        z = torch.randn(T, E, generator=g)
+        z[0] = 0.25                      # all equal: the lowest indices win
+        if E > 2:
+            z[1, 2] = z[1, 0]
+        idx = torch.empty(T, top, dtype=torch.int32, device=device)
+        wts = torch.empty(T, top, dtype=torch.float32, device=device)
+        ops.router_topk(idx, wts, z.to(device), top, 0)
+        for t in range(T):
+            order = sorted(range(E), key=lambda e: (-float(z[t, e]), e))[:top]
+            assert idx[t].tolist() == order, f"row {t}"
+            w = torch.softmax(z[t, order].double(), -1)
+            _close(wts[t], w, "fp32", f"weights of row {t}")
+        ops.router_topk(idx, wts, z.to(device), top, T)
+        assert idx[3].tolist() == [
+            e * T + 3 for e in sorted(range(E),
+                                      key=lambda e: (-float(z[3, e]), e))[:top]]
