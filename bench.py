@@ -38,7 +38,7 @@ def compare_families(args) -> None:
     per token; Rasesun three state-space layers to one latent-attention
     layer with a 1024-token window, every second feed-forward a mixture of
     16 table-routed experts, two active; Dumovik periods of chunk-local
-    attention over 512-token chunks, two linear-attention layers and latent
+    attention over 8192-token chunks, two linear-attention layers and latent
     attention, every second feed-forward a mixture of 16 routed experts, two
     active)."""
     from kukeon_amd.engine.config import (EngineConfig, ModelConfig,
@@ -75,7 +75,7 @@ def compare_families(args) -> None:
             elif fam == "dumovik":
                 cfg = dumovik_bench(width=W, layers=nl, heads=hq,
                                     kv_heads=hk, ff=ff, vocab=vocab,
-                                    chunk=512 if on_gpu else 16,
+                                    chunk=8192 if on_gpu else 16,
                                     experts=16 if on_gpu else 4,
                                     name=f"dumovik-{size}")
             else:

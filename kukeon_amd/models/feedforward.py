@@ -264,7 +264,11 @@ class RoutedMoE(nn.Module):
             ops.clamp_glu(a[at: at + n], z[:, :ff],
                           z[:, self.up_col: self.up_col + ff], None, None,
                           f.limit, self.alpha, 1.0)
-            done[at: at + n] = ops.linear(a[at: at + n], self.w_down[e])
+            if n > 64:      # straight into its rows, no copy
+                torch.mm(a[at: at + n], self.w_down[e].t(),
+                         out=done[at: at + n])
+            else:
+                done[at: at + n] = ops.linear(a[at: at + n], self.w_down[e])
             at += n
         ops.combine_rows_weighted(out, done, inv.view(T, top)
                                   .to(torch.int32), wts)

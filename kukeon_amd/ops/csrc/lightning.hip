@@ -54,11 +54,25 @@ __global__ __launch_bounds__(1024) void lightning_scan_kernel(
   const bool live = e < dv;
   float* st = state + (((long)state_slots[s] * H + h) * dv + (live ? e : 0)) *
                           (long)d + l * NR;
+  // whole 16-byte pieces of the slot when the rows allow it
+  const bool vec4 = (d & 3) == 0;
   float S[NR];
 #pragma unroll
-  for (int i = 0; i < NR; ++i) {
-    const int dd = l * NR + i;
-    S[i] = (live && p0 > 0 && dd < d) ? st[i] : 0.f;
+  for (int i4 = 0; i4 < NR / 4; ++i4) {
+    const int dd = l * NR + 4 * i4;
+    float4 v = float4{0.f, 0.f, 0.f, 0.f};
+    if (live && p0 > 0) {
+      if (vec4) {
+        if (dd < d) v = *reinterpret_cast<const float4*>(st + 4 * i4);
+      } else {
+        if (dd + 0 < d) v.x = st[4 * i4 + 0];
+        if (dd + 1 < d) v.y = st[4 * i4 + 1];
+        if (dd + 2 < d) v.z = st[4 * i4 + 2];
+        if (dd + 3 < d) v.w = st[4 * i4 + 3];
+      }
+    }
+    S[4 * i4 + 0] = v.x; S[4 * i4 + 1] = v.y;
+    S[4 * i4 + 2] = v.z; S[4 * i4 + 3] = v.w;
   }
   const float a = decay[h];
   for (int t0 = 0; t0 < n; t0 += LT_TT) {
@@ -79,13 +93,20 @@ __global__ __launch_bounds__(1024) void lightning_scan_kernel(
     if (live) {
       for (int t = 0; t < nt; ++t) {
         const float v = sV[t * dv + e];
-        const float* kq = sK + t * DP + l * NR;
-        const float* qq = sQ + t * DP + l * NR;
+        const float4* kq =
+            reinterpret_cast<const float4*>(sK + t * DP + l * NR);
+        const float4* qq =
+            reinterpret_cast<const float4*>(sQ + t * DP + l * NR);
         float o = 0.f;
 #pragma unroll
-        for (int i = 0; i < NR; ++i) {
-          S[i] = fmaf(a, S[i], kq[i] * v);
-          o = fmaf(S[i], qq[i], o);
+        for (int i4 = 0; i4 < NR / 4; ++i4) {
+          const float4 k4 = kq[i4];
+          const float4 q4 = qq[i4];
+          float* Si = S + 4 * i4;
+          Si[0] = fmaf(a, Si[0], k4.x * v); o = fmaf(Si[0], q4.x, o);
+          Si[1] = fmaf(a, Si[1], k4.y * v); o = fmaf(Si[1], q4.y, o);
+          Si[2] = fmaf(a, Si[2], k4.z * v); o = fmaf(Si[2], q4.z, o);
+          Si[3] = fmaf(a, Si[3], k4.w * v); o = fmaf(Si[3], q4.w, o);
         }
         for (int off = LN >> 1; off > 0; off >>= 1)
           o += __shfl_xor(o, off, WAVE);
@@ -95,8 +116,18 @@ __global__ __launch_bounds__(1024) void lightning_scan_kernel(
   }
   if (live) {
 #pragma unroll
-    for (int i = 0; i < NR; ++i)
-      if (l * NR + i < d) st[i] = S[i];
+    for (int i4 = 0; i4 < NR / 4; ++i4) {
+      const int dd = l * NR + 4 * i4;
+      if (vec4) {
+        if (dd < d)
+          *reinterpret_cast<float4*>(st + 4 * i4) =
+              float4{S[4 * i4], S[4 * i4 + 1], S[4 * i4 + 2], S[4 * i4 + 3]};
+      } else {
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+          if (dd + j < d) st[4 * i4 + j] = S[4 * i4 + j];
+      }
+    }
   }
 }
 

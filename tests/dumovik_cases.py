@@ -640,6 +640,40 @@ def case_multi_turn(device, dtype):
     assert_greedy(cfg, W, p1 + t1 + p2 + t2 + [7, 3], t3, "rebuilt session")
 
 
+def case_modelhub(device):
+    """The serving daemon's model server with this family: sessions over the
+    unix socket, two turns on one session, greedy tokens as the plain model
+    gives them."""
+    import uuid
+    from kukeon_amd.serve.server import ModelhubClient, ModelhubServer
+    cfg = CONFIGS["hybrid"]()
+    W = weights(cfg, 16)
+    mcfg = DumovikConfig.from_json(cfg)
+    model = DumovikModel(mcfg, device=device, dtype="fp32", tensors=W,
+                         max_position=128)
+    ecfg = EngineConfig(block_size=4, max_model_len=128, max_sessions=4,
+                        state_slots=4, num_kv_blocks=64, use_graphs=False)
+    sock = f"/tmp/mh-{uuid.uuid4().hex[:10]}.sock"
+    hub = ModelhubServer(model, mcfg, ecfg, sock, device=device)
+    hub.start()
+    try:
+        c = ModelhubClient(sock, timeout=120)
+        p1, p2 = tokens(cfg, 6, 70), tokens(cfg, 3, 71)
+        r1 = c.generate("s", p1, max_new_tokens=4, temperature=0.0)
+        assert len(r1["tokens"]) == 4
+        assert_greedy(cfg, W, p1, r1["tokens"], "first turn")
+        r2 = c.generate("s", p2, max_new_tokens=3, temperature=0.0)
+        assert len(r2["tokens"]) == 3
+        assert_greedy(cfg, W, p1 + r1["tokens"] + p2, r2["tokens"],
+                      "second turn")
+        rb = c.generate("t", p2, max_new_tokens=2, temperature=0.0)
+        assert_greedy(cfg, W, p2, rb["tokens"], "other session")
+        assert c.call("stats")["sessions"] == 2
+        c.close()
+    finally:
+        hub.stop()
+
+
 def write_checkpoint(folder, cfg, W):
     """config.json and model.safetensors (8-byte header length, JSON header,
     raw data) of a config dictionary and its tensors."""

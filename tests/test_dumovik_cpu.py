@@ -66,6 +66,10 @@ def test_multi_turn_and_eviction():
     cases.case_multi_turn(DEV, DT)
 
 
+def test_modelhub_serves_the_family():
+    cases.case_modelhub(DEV)
+
+
 def test_checkpoint_folder(tmp_path):
     cases.case_registry(tmp_path, DEV, DT)
 
