@@ -147,7 +147,7 @@ def dumovik_bench(width=4096, layers=8, heads=32, kv_heads=8, ff=14336,
             share = first_attn if (first_attn is not None and
                                    (i // 4) % 2 == 1) else None
             mix = ChunkAttnCfg(heads=heads, kv_heads=kv_heads, dim=128,
-                               vdim=128, scale=128 ** -0.5, softcap=50.0,
+                               vdim=128, scale=128 ** -0.5, softcap=30.0,
                                chunk=chunk, kv_from=share)
             if share is None:
                 first_attn = i
@@ -155,7 +155,7 @@ def dumovik_bench(width=4096, layers=8, heads=32, kv_heads=8, ff=14336,
             kind = "latent_attention"
             mix = LatentAttnCfg(heads=heads, dim=128, rot_dim=64, vdim=128,
                                 q_rank=0, kv_rank=512, scale=192 ** -0.5,
-                                window=0, rot_dims=64, rot_base=500000.0,
+                                window=0, rot_dims=64, rot_base=10000.0,
                                 rot_layout="half", gate="element")
         else:
             kind = "lightning"

@@ -68,14 +68,14 @@ CONFIGS = {
         layer(lightning(), moe(5, 2, 12)),
         layer(latent(), None),
         layer(attn(kv_from=0, chunk=5, softcap=3.0), moe(4, 3, 9)),
-        layer(lightning(heads=2, dim=20, vdim=12, decay=[0.999, 0.3]),
+        layer(lightning(heads=2, dim=20, vdim=12, decay=[0.9975, 0.3]),
               dense(33)),
     ]),
     # rows of whole 16-byte pieces everywhere (the vector forms of the
     # kernels), five query heads on one kv head, six heads on a latent head
     # group of four, one expert per token, state rows spread over lanes
     "aligned": lambda: config([
-        layer(lightning(heads=2, dim=64, vdim=32), moe(4, 1, 64)),
+        layer(lightning(heads=2, dim=64, vdim=40), moe(4, 1, 64)),
         layer(attn(heads=5, kv_heads=1, dim=16, vdim=48, chunk=20),
               dense(128)),
         layer(latent(heads=6, dim=16, rot_dim=8, vdim=16, kv_rank=32),

@@ -36,7 +36,7 @@ def test_op_scan(dtype):
     cases.case_op_scan(DEV, dtype, H=2, d=128, dv=64, cuts=(37, 1, 3))
     # 32 rows per thread, a workgroup of 1024
     cases.case_op_scan(DEV, dtype, H=1, d=128, dv=256, cuts=(5, 18))
-    cases.case_op_scan(DEV, dtype, H=4, d=64, dv=32, cuts=(2, 30, 1, 1))
+    cases.case_op_scan(DEV, dtype, H=3, d=64, dv=24, cuts=(2, 30, 1, 1))
 
 
 def test_op_router():
