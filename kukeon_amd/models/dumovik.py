@@ -334,4 +334,4 @@ class DumovikModel(nn.Module):
         return out
 
     def compute_logits(self, hidden: torch.Tensor) -> torch.Tensor:
-        return ops.linear(hidden, self.embed).float()
+        return ops.linear_f32(hidden, self.embed)

@@ -175,7 +175,7 @@ class RoutedMoE(nn.Module):
     uses the `top` experts with the largest router logits, weighted by the
     softmax over those logits only. Expert: g = min(gate h, limit),
     u = clamp(up h, +-limit), y = g sigmoid(1.702 g) (u + 1), out = down y.
-    The router runs in fp32. Weights are stacked [E, 2 ff', W] (gate rows,
+    The router's logits, the choice and the weights are fp32. Weights are stacked [E, 2 ff', W] (gate rows,
     then up rows, each padded to a multiple of 8) and [E, W, ff].
 
     Two forms behind one call. Few rows (decode steps; nothing leaves the
@@ -206,8 +206,9 @@ class RoutedMoE(nn.Module):
         self.w_down = nn.Parameter(torch.stack(
             [t[p + f"e{e}.down"] for e in range(f.experts)]).to(**dev)
             .contiguous(), requires_grad=False)
-        self.w_router = t[p + "router"].to(device=device,
-                                           dtype=torch.float32).contiguous()
+        # in the activation format: products of two bf16 numbers are exact
+        # in fp32, so the fp32-output GEMM over bf16 rows IS the fp32 router
+        self.w_router = t[p + "router"].to(**dev).contiguous()
 
     @staticmethod
     def tensor_shapes(f: FFCfg, width: int, vocab: int) -> Dict[str, tuple]:
@@ -222,7 +223,7 @@ class RoutedMoE(nn.Module):
                 meta=None) -> torch.Tensor:
         f = self.f
         T, W = h.shape
-        logits = torch.nn.functional.linear(h.float(), self.w_router)
+        logits = ops.linear_f32(h, self.w_router)
         idx = torch.empty(T, f.top, dtype=torch.int32, device=h.device)
         wts = torch.empty(T, f.top, dtype=torch.float32, device=h.device)
         out = torch.empty_like(h)

@@ -298,6 +298,15 @@ def linear(x: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
     return torch.nn.functional.linear(x, w)
 
 
+def linear_f32(x: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
+    """x @ w.T with fp32 OUTPUT: the vendor GEMM accumulates bf16 products
+    in fp32 either way, so keeping the sums unrounded costs nothing. For
+    results that are compared or ranked (logits, router scores)."""
+    if x.is_cuda and x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16:
+        return torch.mm(x, w.t(), out_dtype=torch.float32)
+    return torch.nn.functional.linear(x.float(), w.float())
+
+
 def linear_add_rmsnorm(x: torch.Tensor, w: torch.Tensor,
                        residual: torch.Tensor, norm_weight: torch.Tensor,
                        eps: float) -> torch.Tensor:
