@@ -107,12 +107,14 @@ def build(verbose: bool = True, force: bool = False,
           groups=None) -> Path:
     """Compile and link the given kernel groups (default: all)."""
     out = None
+    done: set = set()       # sources compiled in this call (groups share some)
     for g in (groups or list(GROUPS)):
-        out = _build_group(g, verbose, force)
+        out = _build_group(g, verbose, force, done)
     return out
 
 
-def _build_group(group: str, verbose: bool, force: bool) -> Path:
+def _build_group(group: str, verbose: bool, force: bool,
+                 done: set = None) -> Path:
     modname, sources = GROUPS[group]
     SO_PATH = so_path(group)
     inc, libdirs = _torch_paths()
@@ -146,9 +148,12 @@ def _build_group(group: str, verbose: bool, force: bool) -> Path:
         sp = CSRC / src
         op = OBJ_DIR / (src.rsplit(".", 1)[0] + ".o")
         objs.append(op)
-        if (not force and op.exists()
+        if ((not force or (done is not None and src in done))
+                and op.exists()
                 and op.stat().st_mtime > max(sp.stat().st_mtime, hdr_mtime)):
             continue
+        if done is not None:
+            done.add(src)
         cmd = ["hipcc", "-c", str(sp), "-o", str(op)] + common_flags
         if src.endswith(".cpp"):
             cmd.append("-x")

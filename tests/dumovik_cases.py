@@ -84,13 +84,14 @@ CONFIGS = {
                    softcap=0, kv_from=1), None),
     ], width=128, vocab=50, eps=1e-3),
     # no chunks and no cap (plain causal attention), heads == kv_heads,
-    # every expert chosen, a chunk of one, a decay of exactly one
+    # every expert chosen, a chunk of one, a decay of exactly one, a width
+    # that is not a multiple of 8
     "plain": lambda: config([
         layer(attn(heads=2, kv_heads=2, dim=6, vdim=5, chunk=0, softcap=0),
               moe(3, 3, 10)),
         layer(attn(heads=3, kv_heads=1, dim=4, vdim=4, chunk=1), None),
         layer(lightning(heads=1, dim=5, vdim=7, decay=[1.0]), dense(20)),
-    ], width=24, vocab=31),
+    ], width=26, vocab=31),
     # no attention at all (no cache pages), and no recurrence (no state)
     "only_lightning": lambda: config([
         layer(lightning(heads=2, dim=4, vdim=4), dense(20)),
