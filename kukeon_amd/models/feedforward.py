@@ -13,6 +13,7 @@ import torch
 import torch.nn as nn
 
 from kukeon_amd import ops
+from kukeon_amd.models.mixers import fuse_rows
 
 
 @dataclass
@@ -146,7 +147,6 @@ class GeluGatedFF(nn.Module):
     def __init__(self, f: FFCfg, width: int, t: Dict[str, torch.Tensor],
                  p: str, device, dtype):
         super().__init__()
-        from kukeon_amd.models.mixers import fuse_rows
         self.ff = f.ff
         self.col, self.w_in = fuse_rows(
             [("gate", t[p + "gate"]), ("up", t[p + "up"])], width, dtype,
