@@ -1,0 +1,426 @@
+"""Bezizen: a decoder that carries SEVERAL residual streams. A sublayer reads
+a learned blend of the streams, and its output goes back into every stream
+while the streams are mixed among themselves:
+
+    u     = sum_s in[s] x_s ;  y = sublayer(rmsnorm(u) w)
+    x_j  <- sum_s mix[s, j] x_s + out[j] y          (all j from the old x)
+
+All streams start as the embedding output (token row times a scale plus a
+learned position row); the logits read the sum of the streams after a final
+RMS norm, times a logit scale. A configuration without `streams` keeps the
+plain pre-norm residual x <- x + sublayer(rmsnorm(x) w), which is the same
+machinery with one stream and unit weights.
+
+Layers pick one of two sequence mixers: `wkv` (time mixing with token
+shift, a data-dependent decay per key channel and a bonus for the current
+token) or `parallel` (a sliding-window attention whose values are its keys,
+beside a gated linear attention, their outputs scaled and summed). The
+feed-forward is a mixture of silu-gated experts with a group-limited
+softmax router and a shared expert; a layer may have none.
+
+Everything a checkpoint's config.json states (sizes, the order of layers,
+constants) is read from it. The attention side keeps one key row per token
+in the paged cache; the recurrences, the token-shift row and the
+convolution tails live in the engine's state slots (fp32).
+
+Tensor parallelism is not implemented for this family (tp_size must be 1).
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+from typing import Dict, List, Optional
+
+import torch
+import torch.nn as nn
+
+from kukeon_amd import ops
+from kukeon_amd import parallel
+from kukeon_amd.models.feedforward import FFCfg, RoutedMoE
+from kukeon_amd.models.mixers import (GatedLinearAttention, GatedLinearCfg,
+                                      ParallelMixer, WindowAttention,
+                                      WindowAttnCfg, WkvCfg, WkvMixer)
+
+_DTYPES = {"bf16": torch.bfloat16, "bfloat16": torch.bfloat16,
+           "fp32": torch.float32, "float32": torch.float32}
+
+
+@dataclass
+class ParallelCfg:
+    left: WindowAttnCfg
+    right: GatedLinearCfg
+    left_scale: float
+    right_scale: float
+
+
+@dataclass
+class BezizenLayerCfg:
+    type: str                # "wkv" | "parallel"
+    mixer: object
+    mlp: Optional[FFCfg]
+
+
+@dataclass
+class BezizenConfig:
+    family = "bezizen"
+    name: str = "bezizen"
+    width: int = 1024
+    vocab_size: int = 32000
+    norm_eps: float = 1e-6
+    streams: int = 0         # 0: one plain residual stream
+    embed_scale: float = 1.0
+    logit_scale: float = 1.0
+    max_positions: int = 0   # rows of the learned position table
+    layers: List[BezizenLayerCfg] = field(default_factory=list)
+
+    @property
+    def hidden_size(self) -> int:
+        return self.width
+
+    @property
+    def num_layers(self) -> int:
+        return len(self.layers)
+
+    @property
+    def is_moe(self) -> bool:
+        return False
+
+    @staticmethod
+    def from_json(c: dict, name: str = "bezizen") -> "BezizenConfig":
+        layers = []
+        for i, L in enumerate(c["layers"]):
+            kind = L.get("type")
+            m = L["mixer"]
+            if kind == "wkv":
+                mix = WkvCfg(heads=int(m["heads"]), dim=int(m["dim"]))
+            elif kind == "parallel":
+                a, b = m["left"], m["right"]
+                qt = a.get("q_temp") or {}
+                left = WindowAttnCfg(
+                    heads=int(a["heads"]), kv_heads=int(a["kv_heads"]),
+                    dim=int(a["dim"]), scale=float(a["scale"]),
+                    window=int((a.get("mask") or {}).get("size") or 0),
+                    conv=int(a.get("conv") or 0),
+                    temp_coef=float(qt.get("coef") or 0.0),
+                    temp_every=int(qt.get("every") or 0))
+                if a.get("vdim") is not None and int(a["vdim"]) != left.dim:
+                    raise ValueError(f"layer {i}: values are the keys, so "
+                                     "vdim must equal dim")
+                right = GatedLinearCfg(heads=int(b["heads"]),
+                                       dim=int(b["dim"]),
+                                       vdim=int(b["vdim"]),
+                                       tau=float(b["tau"]))
+                mix = ParallelCfg(left, right,
+                                  float(m.get("left_scale", 1.0)),
+                                  float(m.get("right_scale", 1.0)))
+            else:
+                raise ValueError(f"layer {i}: unknown mixer type {kind!r}")
+            mlp = None
+            if L.get("mlp"):
+                f = L["mlp"]
+                if f.get("kind", "moe") != "moe":
+                    raise ValueError(f"layer {i}: unknown feed-forward kind "
+                                     f"{f.get('kind')!r}")
+                r = f["router"]
+                g = r.get("groups") or {}
+                mlp = FFCfg("moe", int(f["expert"]["ff"]),
+                            experts=int(r["experts"]), top=int(r["top"]),
+                            act="silu", score="all",
+                            groups=int(g.get("count") or 0),
+                            keep=int(g.get("keep") or 0),
+                            route_scale=float(r.get("scale", 1.0)),
+                            shared_ff=int((f.get("shared") or {})
+                                          .get("ff") or 0))
+            layers.append(BezizenLayerCfg(kind, mix, mlp))
+        return BezizenConfig(
+            name=name, width=int(c["width"]), vocab_size=int(c["vocab"]),
+            norm_eps=float(c["norm"]["eps"]),
+            streams=int(c.get("streams") or 0),
+            embed_scale=float((c.get("embedding") or {}).get("scale", 1.0)),
+            logit_scale=float(c.get("logit_scale", 1.0)),
+            max_positions=int(c.get("max_positions") or 0), layers=layers)
+
+
+def bezizen_bench(width=4096, layers=8, heads=32, kv_heads=8, ff=14336,
+                  vocab=128256, window=1024, experts=16, top=2, streams=4,
+                  max_positions=8192, name="bezizen-8b-like"
+                  ) -> BezizenConfig:
+    """A layer stack at real-model sizes (random weights) for throughput
+    runs: three wkv layers (heads of 128) to one parallel layer (windowed
+    attention with heads of 128 beside a gated linear attention over a
+    quarter of the heads); every second feed-forward is absent so that the
+    routed layers carry the dense layer's active width."""
+    ls = []
+    hd = 128 if width >= 1024 else 32
+    for i in range(layers):
+        if i % 4 == 3:
+            kind = "parallel"
+            mix = ParallelCfg(
+                WindowAttnCfg(heads=heads, kv_heads=kv_heads, dim=hd,
+                              scale=hd ** -0.5, window=window, conv=4,
+                              temp_coef=0.1, temp_every=256),
+                GatedLinearCfg(heads=max(1, heads // 4), dim=hd, vdim=hd,
+                               tau=16.0), 1.0, 1.0)
+        else:
+            kind = "wkv"
+            mix = WkvCfg(heads=max(1, width // hd), dim=hd)
+        sh = max(8, ff // 4 // 8 * 8)
+        mlp = FFCfg("moe", max(8, (ff - sh) // top // 8 * 8),
+                    experts=experts, top=top, act="silu", score="all",
+                    groups=4 if experts % 4 == 0 and experts >= 8 else 0,
+                    keep=2 if experts % 4 == 0 and experts >= 8 else 0,
+                    route_scale=1.0, shared_ff=sh)
+        ls.append(BezizenLayerCfg(kind, mix, mlp))
+    return BezizenConfig(name=name, width=width, vocab_size=vocab,
+                         norm_eps=1e-6, streams=streams, embed_scale=1.0,
+                         logit_scale=1.0, max_positions=max_positions,
+                         layers=ls)
+
+
+def _mixer_shapes(L: BezizenLayerCfg, W: int) -> Dict[str, tuple]:
+    if L.type == "wkv":
+        return WkvMixer.tensor_shapes(L.mixer, W)
+    out = {}
+    for n, s in WindowAttention.tensor_shapes(L.mixer.left, W).items():
+        out["left." + n] = s
+    for n, s in GatedLinearAttention.tensor_shapes(L.mixer.right, W).items():
+        out["right." + n] = s
+    return out
+
+
+# low-rank projections whose inner size only the checkpoint states
+_RANK_FREE = (".w1", ".w2", ".a1", ".a2")
+
+
+def tensor_shapes(cfg: BezizenConfig) -> Dict[str, tuple]:
+    """Names and shapes of a checkpoint of this configuration (the inner
+    size of the low-rank decay projections is the checkpoint's to choose;
+    16 here)."""
+    W, S = cfg.width, cfg.streams
+    out = {"embed": (cfg.vocab_size, W)}
+    if cfg.max_positions:
+        out["pos"] = (cfg.max_positions, W)
+    for i, L in enumerate(cfg.layers):
+        p = f"l{i}."
+        subs = ["1"] + (["2"] if L.mlp is not None else [])
+        for q in subs:
+            out[p + "norm" + q] = (W,)
+            if S:
+                out[p + f"hc{q}.in"] = (S,)
+                out[p + f"hc{q}.out"] = (S,)
+                out[p + f"hc{q}.mix"] = (S, S)
+        for n, s in _mixer_shapes(L, W).items():
+            out[p + "mix." + n] = s
+        if L.mlp is not None:
+            for n, s in RoutedMoE.tensor_shapes(L.mlp, W,
+                                                cfg.vocab_size).items():
+                out[p + "mlp." + n] = s
+    out["final.norm"] = (W,)
+    out["head"] = (cfg.vocab_size, W)
+    return out
+
+
+def random_tensors(cfg: BezizenConfig, seed: int = 0,
+                   device="cpu") -> Dict[str, torch.Tensor]:
+    """Random bf16 weights at a scale that keeps activations O(1)."""
+    on_gpu = torch.device(device).type == "cuda"
+    gdev = device if on_gpu else "cpu"
+    g = torch.Generator(device=gdev).manual_seed(seed)
+    S = max(cfg.streams, 1)
+    out = {}
+
+    def rn(shp, std=1.0, mean=0.0):
+        return mean + torch.randn(shp, generator=g, device=gdev) * std
+
+    for name, shp in tensor_shapes(cfg).items():
+        leaf = name.rsplit(".", 1)[-1]
+        if ".hc" in name:
+            if leaf == "mix":
+                t = torch.eye(S, device=gdev) + rn(shp, 0.1)
+            elif leaf == "in":
+                t = rn(shp, 0.1, 1.0 / S)
+            else:
+                t = rn(shp, 0.1, 1.0)
+        elif ".mu." in name:
+            t = torch.rand(shp, generator=g, device=gdev)
+        elif name.endswith(".conv"):
+            t = rn(shp, 0.3, 1.0 / shp[1])
+        elif leaf == "w0":
+            t = rn(shp, 0.5, -1.0)
+        elif name.endswith("a2.b"):
+            t = rn(shp, 0.5, 2.0)
+        elif leaf == "u":
+            t = rn(shp, 0.3)
+        elif name == "pos":
+            t = rn(shp, 0.1)
+        elif len(shp) == 2:
+            std = shp[1] ** -0.5 if name != "embed" else 1.0
+            if leaf == "router":
+                std *= 2.0
+            t = rn(shp, std)
+        elif leaf in ("norm1", "norm2"):
+            t = rn(shp, 0.1, 0.5)
+        else:
+            t = rn(shp, 0.1, 1.0)
+        out[name] = t.to(torch.bfloat16).to(device)
+    return out
+
+
+class StreamPort:
+    """One sublayer's read and write weights over the streams (fp32)."""
+
+    def __init__(self, t, p: str, streams: int, device):
+        f32 = dict(device=device, dtype=torch.float32)
+        if streams:
+            self.read = t[p + "in"].to(**f32).contiguous()
+            self.mix = t[p + "mix"].to(**f32).contiguous()
+            self.out = t[p + "out"].to(**f32).contiguous()
+        else:
+            self.read = torch.ones(1, **f32)
+            self.mix = torch.ones(1, 1, **f32)
+            self.out = torch.ones(1, **f32)
+
+
+class BezizenLayer(nn.Module):
+    def __init__(self, cfg: BezizenConfig, idx: int,
+                 t: Dict[str, torch.Tensor], device, dtype):
+        super().__init__()
+        L = cfg.layers[idx]
+        p = f"l{idx}."
+        W, eps = cfg.width, cfg.norm_eps
+        f32 = dict(device=device, dtype=torch.float32)
+        self.norm1 = t[p + "norm1"].to(**f32).contiguous()
+        self.port1 = StreamPort(t, p + "hc1.", cfg.streams, device)
+        if L.type == "wkv":
+            self.mixer = WkvMixer(L.mixer, W, eps, t, p + "mix.", device,
+                                  dtype)
+        else:
+            m = L.mixer
+            self.mixer = ParallelMixer(
+                WindowAttention(m.left, W, eps, t, p + "mix.left.", device,
+                                dtype),
+                GatedLinearAttention(m.right, W, eps, t, p + "mix.right.",
+                                     device, dtype),
+                m.left_scale, m.right_scale)
+        self.ff = None
+        if L.mlp is not None:
+            self.norm2 = t[p + "norm2"].to(**f32).contiguous()
+            self.port2 = StreamPort(t, p + "hc2.", cfg.streams, device)
+            self.ff = RoutedMoE(L.mlp, W, t, p + "mlp.", device, dtype)
+
+
+class BezizenModel(nn.Module):
+    family = "bezizen"
+    op_groups = ("strm",)       # kernel groups the forward pass needs
+
+    def __init__(self, cfg: BezizenConfig, device="cuda", dtype="bf16",
+                 tensors: Optional[Dict[str, torch.Tensor]] = None,
+                 max_position: int = 4096, seed: int = 0):
+        super().__init__()
+        if parallel.tp_size() != 1:
+            raise NotImplementedError("Bezizen runs with tp_size == 1 only")
+        self.cfg = cfg
+        self.device_ = torch.device(device)
+        self.dtype = _DTYPES[dtype] if isinstance(dtype, str) else dtype
+        if tensors is None:
+            tensors = random_tensors(cfg, seed, device=self.device_)
+        for name, shp in tensor_shapes(cfg).items():
+            if name not in tensors:
+                raise KeyError(f"checkpoint lacks tensor {name}")
+            got = tuple(tensors[name].shape)
+            if name.endswith(_RANK_FREE) and len(got) == 2:
+                # [rank, W] / [C, rank]: the rank is read from the tensor
+                fixed = 1 if name.endswith(("1",)) else 0
+                if got[fixed] != shp[fixed]:
+                    raise ValueError(f"{name}: shape {got}")
+                continue
+            if got != tuple(shp):
+                raise ValueError(f"{name}: shape {got}, configuration says "
+                                 f"{tuple(shp)}")
+        dev, dt = self.device_, self.dtype
+        self.embed = nn.Parameter(tensors["embed"].to(dev).to(dt),
+                                  requires_grad=False)
+        self.pos = (nn.Parameter(tensors["pos"].to(dev).to(dt),
+                                 requires_grad=False)
+                    if cfg.max_positions else None)
+        self.head = nn.Parameter(tensors["head"].to(dev).to(dt).contiguous(),
+                                 requires_grad=False)
+        self.layers = nn.ModuleList(
+            [BezizenLayer(cfg, i, tensors, dev, dt)
+             for i in range(cfg.num_layers)])
+        self.final_norm = tensors["final.norm"].to(dev).float().contiguous()
+        self.sum_read = torch.ones(max(cfg.streams, 1), dtype=torch.float32,
+                                   device=dev)
+        self.max_position = cfg.max_positions or max_position
+
+    @classmethod
+    def from_checkpoint(cls, model_dir: str, device="cuda", dtype="bf16",
+                        max_position: int = 4096):
+        from kukeon_amd.models.weights import read_checkpoint
+        config, tensors = read_checkpoint(model_dir)
+        cfg = BezizenConfig.from_json(config)
+        return cfg, cls(cfg, device=device, dtype=dtype, tensors=tensors,
+                        max_position=max_position)
+
+    def set_max_position(self, n: int) -> None:
+        """Positions are rows of a learned table: there is nothing to
+        rebuild, and the table bounds the longest sequence."""
+        self.max_position = min(n, self.cfg.max_positions or n)
+
+    # ---- what the engine asks of a model with its own cache layout ----
+    def kv_specs(self):
+        return [L.mixer.kv_spec() for L in self.layers]
+
+    def state_shapes(self):
+        return [L.mixer.state_shape() for L in self.layers]
+
+    def activation_dtype(self) -> torch.dtype:
+        return self.dtype
+
+    # ---- forward ----
+    def forward(self, input_ids: torch.Tensor, kv_k, kv_v, meta,
+                taps: Optional[list] = None) -> torch.Tensor:
+        """-> final-normed hidden [T, W]. `taps`, if a list, receives the
+        sum of the fp32 streams after every layer."""
+        cfg = self.cfg
+        eps = cfg.norm_eps
+        T = input_ids.shape[0]
+        dev = input_ids.device
+        xs = torch.empty(T, max(cfg.streams, 1), cfg.width,
+                         dtype=torch.float32, device=dev)
+        ops.embed_streams(xs, input_ids, meta.positions, self.embed, self.pos,
+                          cfg.embed_scale)
+        h = torch.empty(T, cfg.width, dtype=self.dtype, device=dev)
+        first = self.layers[0]
+        ops.stream_read_norm(h, xs, first.port1.read, first.norm1, eps)
+        n = len(self.layers)
+        for i, layer in enumerate(self.layers):
+            if i + 1 < n:
+                nxt = self.layers[i + 1]
+                nread, nnorm = nxt.port1.read, nxt.norm1
+            else:
+                nread, nnorm = self.sum_read, self.final_norm
+            st = meta.state[i] if meta.state is not None else None
+            y = layer.mixer(h, kv_k[i], st, meta, kv_v[i])
+            h = torch.empty_like(h)
+            if layer.ff is not None:
+                ops.stream_write_read_norm(xs, y, layer.port1.mix,
+                                           layer.port1.out, layer.port2.read,
+                                           layer.norm2, eps, h)
+                y = layer.ff(h, input_ids, meta)
+                h = torch.empty_like(h)
+                ops.stream_write_read_norm(xs, y, layer.port2.mix,
+                                           layer.port2.out, nread, nnorm, eps,
+                                           h)
+            else:
+                ops.stream_write_read_norm(xs, y, layer.port1.mix,
+                                           layer.port1.out, nread, nnorm, eps,
+                                           h)
+            if taps is not None:
+                taps.append(xs.sum(1))
+        return h
+
+    def compute_logits(self, hidden: torch.Tensor) -> torch.Tensor:
+        logits = ops.linear_f32(hidden, self.head)
+        if self.cfg.logit_scale != 1.0:
+            logits = logits * self.cfg.logit_scale
+        return logits

@@ -23,6 +23,17 @@ class FFCfg:
     experts: int = 0
     top: int = 0
     limit: float = 0.0       # clamp of the routed experts' gate and up
+    # routed experts: "clamp" is g sigmoid(1.702 g) (u + 1) with g and u
+    # clamped to `limit`; "silu" is silu(g) u
+    act: str = "clamp"
+    # "top": weights = softmax over the chosen logits; "all": scores =
+    # softmax over all logits, the chosen scores divided by their sum and
+    # multiplied by route_scale
+    score: str = "top"
+    groups: int = 0          # experts in this many equal runs of neighbours,
+    keep: int = 0            # of which only the best `keep` can be chosen
+    route_scale: float = 1.0
+    shared_ff: int = 0       # hidden size of an always-on expert (0: none)
 
 
 def _softplus(x: float) -> float:
@@ -175,7 +186,14 @@ class RoutedMoE(nn.Module):
     uses the `top` experts with the largest router logits, weighted by the
     softmax over those logits only. Expert: g = min(gate h, limit),
     u = clamp(up h, +-limit), y = g sigmoid(1.702 g) (u + 1), out = down y.
-    The router's logits, the choice and the weights are fp32. Weights are stacked [E, 2 ff', W] (gate rows,
+    The router's logits, the choice and the weights are fp32.
+
+    Variants by configuration: experts of the form down(silu(gate h) up h)
+    (`act`); scores from a softmax over ALL logits, the chosen ones divided
+    by their sum and scaled, the choice limited to the best `keep` of
+    `groups` runs of neighbouring experts (`score`, `groups`); an always-on
+    shared expert of the same form (`shared_ff`), which enters the fold as
+    one more chosen row with weight 1. Weights are stacked [E, 2 ff', W] (gate rows,
     then up rows, each padded to a multiple of 8) and [E, W, ff].
 
     Two forms behind one call. Few rows (decode steps; nothing leaves the
@@ -194,8 +212,30 @@ class RoutedMoE(nn.Module):
         super().__init__()
         if not (0 < f.top <= f.experts):
             raise ValueError(f"{p}: top must be within 1 .. experts")
+        if f.act not in ("clamp", "silu") or f.score not in ("top", "all"):
+            raise ValueError(f"{p}: unknown expert or router kind")
+        if f.groups:
+            if f.score != "all" or f.experts % f.groups or \
+                    not (0 < f.keep <= f.groups) or \
+                    f.top > f.keep * (f.experts // f.groups):
+                raise ValueError(f"{p}: expert groups do not fit the router")
         self.f = f
+        # clamp_glu's constants: the silu form is the unclamped one with
+        # alpha 1 and no shift
+        self.glu = ((f.limit, self.alpha, 1.0) if f.act == "clamp"
+                    else (float("inf"), 1.0, 0.0))
         dev = dict(device=device, dtype=dtype)
+        self.shared = None
+        if f.shared_ff:
+            sp = (f.shared_ff + 7) // 8 * 8
+            sgu = torch.zeros(2 * sp, width, **dev)
+            sgu[:f.shared_ff] = t[p + "shared.gate"].to(**dev)
+            sgu[sp: sp + f.shared_ff] = t[p + "shared.up"].to(**dev)
+            self.shared = (nn.Parameter(sgu.contiguous(),
+                                        requires_grad=False),
+                           nn.Parameter(t[p + "shared.down"].to(**dev)
+                                        .contiguous(), requires_grad=False),
+                           sp)
         pad = (f.ff + 7) // 8 * 8
         self.up_col = pad
         gu = torch.zeros(f.experts, 2 * pad, width, **dev)
@@ -217,44 +257,97 @@ class RoutedMoE(nn.Module):
             out[f"e{e}.gate"] = (f.ff, width)
             out[f"e{e}.up"] = (f.ff, width)
             out[f"e{e}.down"] = (width, f.ff)
+        if f.shared_ff:
+            out.update({"shared.gate": (f.shared_ff, width),
+                        "shared.up": (f.shared_ff, width),
+                        "shared.down": (width, f.shared_ff)})
         return out
+
+    def _route(self, idx, wts, logits, dense_rows: int) -> None:
+        """Fill the first `top` columns of idx and wts."""
+        f = self.f
+        if f.score == "all":
+            ops.router_select(idx, wts, logits, f.top, f.groups, f.keep,
+                              f.route_scale, dense_rows)
+        elif idx.shape[1] == f.top:
+            ops.router_topk(idx, wts, logits, f.top, dense_rows)
+        else:
+            i2 = torch.empty(idx.shape[0], f.top, dtype=idx.dtype,
+                             device=idx.device)
+            w2 = torch.empty(idx.shape[0], f.top, dtype=wts.dtype,
+                             device=idx.device)
+            ops.router_topk(i2, w2, logits, f.top, dense_rows)
+            idx[:, :f.top] = i2
+            wts[:, :f.top] = w2
+
+    def _shared_into(self, dst, h) -> None:
+        """dst [T, W] = the shared expert's output."""
+        w_gu, w_down, sp = self.shared
+        ff = self.f.shared_ff
+        z = ops.linear(h, w_gu)
+        a = torch.empty(h.shape[0], ff, dtype=h.dtype, device=h.device)
+        ops.clamp_glu(a, z[:, :ff], z[:, sp: sp + ff], None, None, *self.glu)
+        if h.shape[0] > 64:
+            torch.mm(a, w_down.t(), out=dst)
+        else:
+            dst.copy_(ops.linear(a, w_down))
 
     def forward(self, h: torch.Tensor, ids: torch.Tensor,
                 meta=None) -> torch.Tensor:
         f = self.f
         T, W = h.shape
         logits = ops.linear_f32(h, self.w_router)
-        idx = torch.empty(T, f.top, dtype=torch.int32, device=h.device)
-        wts = torch.empty(T, f.top, dtype=torch.float32, device=h.device)
+        # with a shared expert the fold takes one more row per token
+        cols = f.top + (1 if self.shared is not None else 0)
+        idx = torch.empty(T, cols, dtype=torch.int32, device=h.device)
+        wts = torch.empty(T, cols, dtype=torch.float32, device=h.device)
         out = torch.empty_like(h)
         on_host = getattr(meta, "host_ids", None) is not None
         if on_host and T >= self.sorted_min_rows:
-            ops.router_topk(idx, wts, logits, f.top, 0)
+            self._route(idx, wts, logits, 0)
             return self._forward_sorted(out, h, idx, wts)
         # every expert over every row; idx names rows of the [E*T, W] result
-        ops.router_topk(idx, wts, logits, f.top, T)
+        self._route(idx, wts, logits, T)
         E, ff = f.experts, f.ff
         z = torch.bmm(h.unsqueeze(0).expand(E, T, W),
                       self.w_gu.transpose(1, 2)).view(E * T, -1)
         a = torch.empty(E * T, ff, dtype=h.dtype, device=h.device)
         ops.clamp_glu(a, z[:, :ff], z[:, self.up_col: self.up_col + ff],
-                      None, None, f.limit, self.alpha, 1.0)
-        y = torch.bmm(a.view(E, T, ff), self.w_down.transpose(1, 2))
-        ops.combine_rows_weighted(out, y.view(E * T, W), idx, wts)
+                      None, None, *self.glu)
+        y = torch.empty((E + 1) * T if self.shared is not None else E * T, W,
+                        dtype=h.dtype, device=h.device)
+        torch.bmm(a.view(E, T, ff), self.w_down.transpose(1, 2),
+                  out=y[: E * T].view(E, T, W))
+        if self.shared is not None:
+            self._shared_into(y[E * T:], h)
+            idx[:, f.top] = self._arange(T, h.device) + E * T
+            wts[:, f.top] = 1.0
+        ops.combine_rows_weighted(out, y, idx, wts)
         return out
+
+    def _arange(self, n: int, device) -> torch.Tensor:
+        """0 .. n-1 as int32, kept so that a captured step allocates and
+        fills nothing new."""
+        a = getattr(self, "_ar", None)
+        if a is None or a.numel() < n or a.device != device:
+            a = self._ar = torch.arange(max(n, 64), dtype=torch.int32,
+                                        device=device)
+        return a[:n]
 
     def _forward_sorted(self, out, h, idx, wts) -> torch.Tensor:
         f = self.f
         T, W = h.shape
         E, ff, top = f.experts, f.ff, f.top
-        flat = idx.view(-1).long()
+        flat = idx[:, :top].reshape(-1).long()
         order = torch.argsort(flat, stable=True)
         counts = torch.bincount(flat, minlength=E).tolist()  # host sync
         inv = torch.empty_like(order)
         inv[order] = torch.arange(order.numel(), device=h.device)
         rows = torch.empty(T * top, W, dtype=h.dtype, device=h.device)
         ops.gather_rows(rows, h, (order // top).to(torch.int32))
-        done = torch.empty_like(rows)
+        shared = self.shared is not None
+        done = torch.empty(T * (top + 1) if shared else T * top, W,
+                           dtype=h.dtype, device=h.device)
         a = torch.empty(T * top, ff, dtype=h.dtype, device=h.device)
         at = 0
         for e in range(E):
@@ -264,13 +357,20 @@ class RoutedMoE(nn.Module):
             z = ops.linear(rows[at: at + n], self.w_gu[e])
             ops.clamp_glu(a[at: at + n], z[:, :ff],
                           z[:, self.up_col: self.up_col + ff], None, None,
-                          f.limit, self.alpha, 1.0)
+                          *self.glu)
             if n > 64:      # straight into its rows, no copy
                 torch.mm(a[at: at + n], self.w_down[e].t(),
                          out=done[at: at + n])
             else:
                 done[at: at + n] = ops.linear(a[at: at + n], self.w_down[e])
             at += n
+        if shared:
+            self._shared_into(done[T * top:], h)
+            idx[:, :top] = inv.view(T, top).to(torch.int32)
+            idx[:, top] = self._arange(T, h.device) + T * top
+            wts[:, top] = 1.0
+            ops.combine_rows_weighted(out, done, idx, wts)
+            return out
         ops.combine_rows_weighted(out, done, inv.view(T, top)
                                   .to(torch.int32), wts)
         return out

@@ -450,3 +450,375 @@ class LightningMixer(nn.Module):
         ops.gated_rmsnorm(g, y, proj[:, c["g"]: c["g"] + inner], self.norm_w,
                           self.eps)
         return ops.linear(g, self.w_o)
+
+
+# ---------------------------------------------------------------------------
+@dataclass
+class WkvCfg:
+    heads: int
+    dim: int                 # key channels = value channels per head
+
+
+class WkvMixer(nn.Module):
+    """Time mixing with a data-dependent decay per key channel and a bonus
+    for the current token. Each of r, k, v, g, w reads its own blend of the
+    input h and the previous token's input h', h + (h' - h) mu; r, k, v are
+    projections of their blends, the output gate is silu of g's projection,
+    and the decay is exp(-exp(W2 tanh(W1 blend_w) + w0)). Per head, with the
+    state S [key channel, value channel]:
+
+        o_t = (S_(t-1) + diag(u) k_t v_t^T)^T r_t
+        S_t = diag(decay_t) S_(t-1) + k_t v_t^T
+
+    Each head's o is divided by its root mean square, then weight, gate and
+    output projection. Carried per sequence (fp32 state slots): h' and S^T.
+
+    Tensors (prefix p): mu.{r,k,v,g,w} [W], r, k, v, g [H*dim, W],
+    w1 [rank, W], w2 [H*dim, rank], w0 [H*dim], u [H, dim], norm [H*dim],
+    o [W, H*dim]."""
+
+    BLENDS = ("r", "k", "v", "g", "w")
+
+    def __init__(self, m: WkvCfg, width: int, eps: float,
+                 t: Dict[str, torch.Tensor], p: str, device, dtype):
+        super().__init__()
+        self.m = m
+        self.eps = eps
+        f32 = dict(device=device, dtype=torch.float32)
+        dev = dict(device=device, dtype=dtype)
+        self.mu = torch.stack([t[p + "mu." + n] for n in self.BLENDS]).to(
+            **f32).contiguous()
+        # r, k, v, g have one shape: one batched GEMM over their blends
+        self.w_rkvg = nn.Parameter(torch.stack(
+            [t[p + n] for n in ("r", "k", "v", "g")]).to(**dev).contiguous(),
+            requires_grad=False)
+        self.w1 = nn.Parameter(t[p + "w1"].to(**dev).contiguous(),
+                               requires_grad=False)
+        self.w2 = nn.Parameter(t[p + "w2"].to(**dev).contiguous(),
+                               requires_grad=False)
+        self.w0 = t[p + "w0"].to(**f32).contiguous()
+        self.bonus = t[p + "u"].to(**f32).reshape(-1).contiguous()
+        self.norm_w = t[p + "norm"].to(**f32).contiguous()
+        self.w_o = nn.Parameter(t[p + "o"].to(**dev).contiguous(),
+                                requires_grad=False)
+
+    @staticmethod
+    def tensor_shapes(m: WkvCfg, width: int, rank: int = 16):
+        C = m.heads * m.dim
+        out = {"mu." + n: (width,) for n in WkvMixer.BLENDS}
+        out.update({n: (C, width) for n in ("r", "k", "v", "g")})
+        out.update({"w1": (rank, width), "w2": (C, rank), "w0": (C,),
+                    "u": (m.heads, m.dim), "norm": (C,), "o": (width, C)})
+        return out
+
+    def kv_spec(self) -> Optional[LayerKVSpec]:
+        return None
+
+    def state_shape(self):
+        m = self.m
+        return [(self.mu.shape[1],), (m.heads, m.dim, m.dim)]
+
+    @property
+    def out_width(self) -> int:
+        return self.m.heads * self.m.dim
+
+    def forward(self, h: torch.Tensor, cache, state, meta,
+                cache_v=None) -> torch.Tensor:
+        g = torch.empty(h.shape[0], self.out_width, dtype=h.dtype,
+                        device=h.device)
+        self.pre_output(h, cache, state, meta, cache_v, g, 1.0)
+        return ops.linear(g, self.w_o)
+
+    def pre_output(self, h, cache, state, meta, cache_v, out,
+                   scale: float) -> None:
+        """The input of the output projection, times `scale`, into `out`."""
+        m = self.m
+        T, W = h.shape
+        C = m.heads * m.dim
+        prev, S = state
+        one = meta.max_rows == 1 and T == meta.cu_rows.numel() - 1
+        blends = torch.empty(5, T, W, dtype=h.dtype, device=h.device)
+        ops.token_shift(blends, h, self.mu, prev, meta.positions,
+                        meta.row_seq, meta.cu_rows, meta.state_slots, one)
+        if not one:
+            ops.token_shift_tail(prev, h, meta.positions, meta.cu_rows,
+                                 meta.state_slots)
+        rkvg = torch.bmm(blends[:4], self.w_rkvg.transpose(1, 2))  # [4,T,C]
+        lo = ops.linear_f32(blends[4], self.w1)
+        lo_t = torch.empty(lo.shape, dtype=h.dtype, device=h.device)
+        ops.tanh_cast(lo_t, lo)
+        z = ops.linear_f32(lo_t, self.w2)                          # [T, C]
+        y = torch.empty(T, C, dtype=torch.float32, device=h.device)
+        ops.decay_scan(y, rkvg[0], rkvg[1], rkvg[2], z, self.w0, self.bonus,
+                       S, meta.positions, meta.cu_rows, meta.state_slots,
+                       m.heads, m.dim, m.dim, 0)
+        ops.head_rmsnorm_gate(out, y, rkvg[3], self.norm_w, m.heads,
+                              self.eps, 0, scale)
+
+
+# ---------------------------------------------------------------------------
+@dataclass
+class WindowAttnCfg:
+    heads: int
+    kv_heads: int
+    dim: int                 # query/key entries per head; values = keys
+    scale: float
+    window: int = 0          # position i sees i-window+1 .. i (0: all)
+    conv: int = 0            # taps of the convolution on q and k (0: none)
+    temp_coef: float = 0.0   # queries times 1 + coef ln(floor((p+1)/every)+1)
+    temp_every: int = 0      # (0: no temperature)
+    bias: bool = True        # slope_h (i - j) off the scores
+
+
+def distance_slopes(heads: int) -> torch.Tensor:
+    """slope_h = 2^(-8 (h + 1) / heads)."""
+    return torch.tensor([2.0 ** (-8.0 * (h + 1) / heads)
+                         for h in range(heads)], dtype=torch.float64)
+
+
+class WindowAttention(nn.Module):
+    """Grouped-query softmax attention over a sliding window whose values
+    are its keys (one cache row per token and kv head). q and k pass a short
+    causal convolution per channel straight after their projections; there
+    is no rotation: positions enter through a query temperature that grows
+    with the logarithm of the position, and through a bias slope_h (i - j)
+    taken off the scaled scores. The concatenated heads are multiplied by
+    sigmoid of a gate projected from the mixer's input, then projected out.
+    Carried per sequence: the last taps-1 projected q and k rows (fp32).
+
+    Tensors (prefix p): q [H*dim, W], k [G*dim, W], q.conv [H*dim, taps],
+    k.conv [G*dim, taps], g [H*dim, W], o [W, H*dim]."""
+
+    def __init__(self, m: WindowAttnCfg, width: int, eps: float,
+                 t: Dict[str, torch.Tensor], p: str, device, dtype):
+        super().__init__()
+        if m.heads % m.kv_heads:
+            raise ValueError(f"{p}: heads not a multiple of kv_heads")
+        self.m = m
+        self.Cq, self.Ck = m.heads * m.dim, m.kv_heads * m.dim
+        self.col, self.w_in = fuse_rows(
+            [("q", t[p + "q"]), ("k", t[p + "k"]), ("g", t[p + "g"])], width,
+            dtype, device)
+        f32 = dict(device=device, dtype=torch.float32)
+        taps = max(1, m.conv)
+        if m.conv:
+            cw = torch.cat([t[p + "q.conv"], t[p + "k.conv"]], 0)
+            if tuple(cw.shape) != (self.Cq + self.Ck, taps):
+                raise ValueError(f"{p}: convolution shape {tuple(cw.shape)}")
+            self.conv_w = cw.to(**f32).t().contiguous()       # [taps, C]
+        else:
+            self.conv_w = torch.ones(1, self.Cq + self.Ck, **f32)
+        self.taps = taps
+        self.zero_b = torch.zeros(self.Cq + self.Ck, **f32)
+        self.slopes = (distance_slopes(m.heads).to(**f32).contiguous()
+                       if m.bias else None)
+        self.w_o = nn.Parameter(t[p + "o"].to(device=device, dtype=dtype)
+                                .contiguous(), requires_grad=False)
+
+    @staticmethod
+    def tensor_shapes(m: WindowAttnCfg, width: int) -> Dict[str, tuple]:
+        Cq, Ck = m.heads * m.dim, m.kv_heads * m.dim
+        out = {"q": (Cq, width), "k": (Ck, width), "g": (Cq, width),
+               "o": (width, Cq)}
+        if m.conv:
+            out.update({"q.conv": (Cq, m.conv), "k.conv": (Ck, m.conv)})
+        return out
+
+    def kv_spec(self) -> Optional[LayerKVSpec]:
+        return LayerKVSpec(self.m.kv_heads, self.m.dim, 0)
+
+    def state_shape(self):
+        return (self.taps - 1, self.Cq + self.Ck)
+
+    @property
+    def out_width(self) -> int:
+        return self.Cq
+
+    def forward(self, h: torch.Tensor, cache, state, meta,
+                cache_v=None) -> torch.Tensor:
+        og = torch.empty(h.shape[0], self.Cq, dtype=h.dtype, device=h.device)
+        self.pre_output(h, cache, state, meta, cache_v, og, 1.0)
+        return ops.linear(og, self.w_o)
+
+    def pre_output(self, h, cache, state, meta, cache_v, out,
+                   scale: float) -> None:
+        m = self.m
+        T = h.shape[0]
+        c = self.col
+        proj = ops.linear(h, self.w_in)
+        q = torch.empty(T, self.Cq, dtype=h.dtype, device=h.device)
+        one = meta.max_rows == 1 and T == meta.cu_rows.numel() - 1
+        ops.conv_scale_append(q, cache, proj, c["q"], c["k"], self.conv_w,
+                              state, m.temp_coef, m.temp_every,
+                              meta.positions, meta.row_seq, meta.cu_rows,
+                              meta.state_slots, meta.block_table, one)
+        if not one and self.taps > 1:
+            ops.conv_pair_tail_update(state, proj, c["q"], c["k"], self.Cq,
+                                      self.Ck, self.zero_b, meta.positions,
+                                      meta.cu_rows, meta.state_slots)
+        o = torch.empty(T, self.Cq, dtype=h.dtype, device=h.device)
+        if (meta.mode == "prefill" and meta.max_rows >= 16 and
+                meta.qb_seq is not None and
+                ops.window_tiles_supported(q, m.dim, cache.shape[2])):
+            # prompt portions on the matrix cores
+            ops.window_attention_tiles(o, q, cache, self.slopes,
+                                       meta.block_table, meta.seq_lens,
+                                       meta.q_starts, meta.qb_seq,
+                                       meta.qb_start, m.scale, m.window)
+        else:
+            ops.window_attention(o, q, cache, None, self.slopes,
+                                 meta.positions, meta.row_seq,
+                                 meta.block_table, m.heads, m.scale, m.window)
+        ops.scaled_gate(out, o, proj[:, c["g"]: c["g"] + self.Cq], 1, scale)
+
+
+# ---------------------------------------------------------------------------
+@dataclass
+class GatedLinearCfg:
+    heads: int
+    dim: int
+    vdim: int
+    tau: float               # decay = sigmoid(z)^(1/tau)
+
+
+class GatedLinearAttention(nn.Module):
+    """Linear attention with a learned decay per key channel:
+    q = W_q h dim^(-1/2), k = W_k h, v = W_v h,
+    decay_t = sigmoid(W_a2 (W_a1 h) + b)^(1/tau), and per head
+
+        S_t = diag(decay_t) S_(t-1) + k_t v_t^T ,  o_t = S_t^T q_t .
+
+    Each head's o is RMS-normed over its value entries with one weight
+    vector shared by the heads, the concatenation is multiplied by
+    silu(W_g h) and projected out. Carried per sequence: S^T (fp32).
+
+    Tensors (prefix p): q, k [H*dim, W], v, g [H*vdim, W], a1 [rank, W],
+    a2 [H*dim, rank], a2.b [H*dim], norm [vdim], o [W, H*vdim]."""
+
+    def __init__(self, m: GatedLinearCfg, width: int, eps: float,
+                 t: Dict[str, torch.Tensor], p: str, device, dtype):
+        super().__init__()
+        self.m = m
+        self.eps = eps
+        self.col, self.w_in = fuse_rows(
+            [("q", t[p + "q"]), ("k", t[p + "k"]), ("v", t[p + "v"]),
+             ("g", t[p + "g"]), ("a", t[p + "a1"])], width, dtype, device)
+        self.rank = t[p + "a1"].shape[0]
+        f32 = dict(device=device, dtype=torch.float32)
+        self.w_a2 = nn.Parameter(t[p + "a2"].to(device=device, dtype=dtype)
+                                 .contiguous(), requires_grad=False)
+        self.a_bias = t[p + "a2.b"].to(**f32).contiguous()
+        self.norm_w = t[p + "norm"].to(**f32).repeat(m.heads).contiguous()
+        self.w_o = nn.Parameter(t[p + "o"].to(device=device, dtype=dtype)
+                                .contiguous(), requires_grad=False)
+
+    @staticmethod
+    def tensor_shapes(m: GatedLinearCfg, width: int, rank: int = 16):
+        H = m.heads
+        return {"q": (H * m.dim, width), "k": (H * m.dim, width),
+                "v": (H * m.vdim, width), "g": (H * m.vdim, width),
+                "a1": (rank, width), "a2": (H * m.dim, rank),
+                "a2.b": (H * m.dim,), "norm": (m.vdim,),
+                "o": (width, H * m.vdim)}
+
+    def kv_spec(self) -> Optional[LayerKVSpec]:
+        return None
+
+    def state_shape(self):
+        return (self.m.heads, self.m.vdim, self.m.dim)
+
+    @property
+    def out_width(self) -> int:
+        return self.m.heads * self.m.vdim
+
+    def forward(self, h: torch.Tensor, cache, state, meta,
+                cache_v=None) -> torch.Tensor:
+        g = torch.empty(h.shape[0], self.out_width, dtype=h.dtype,
+                        device=h.device)
+        self.pre_output(h, cache, state, meta, cache_v, g, 1.0)
+        return ops.linear(g, self.w_o)
+
+    def pre_output(self, h, cache, state, meta, cache_v, out,
+                   scale: float) -> None:
+        m = self.m
+        T = h.shape[0]
+        c = self.col
+        Cq, Cv = m.heads * m.dim, m.heads * m.vdim
+        proj = ops.linear(h, self.w_in)
+        z = ops.linear_f32(proj[:, c["a"]: c["a"] + self.rank], self.w_a2)
+        y = torch.empty(T, Cv, dtype=torch.float32, device=h.device)
+        ops.decay_scan(y, proj[:, c["q"]: c["q"] + Cq],
+                       proj[:, c["k"]: c["k"] + Cq],
+                       proj[:, c["v"]: c["v"] + Cv], z, self.a_bias, None,
+                       state, meta.positions, meta.cu_rows, meta.state_slots,
+                       m.heads, m.dim, m.vdim, 1, m.tau, m.dim ** -0.5)
+        ops.head_rmsnorm_gate(out, y, proj[:, c["g"]: c["g"] + Cv],
+                              self.norm_w, m.heads, self.eps, 0, scale)
+
+
+# ---------------------------------------------------------------------------
+class ParallelMixer(nn.Module):
+    """Two mixers side by side on the same input; the result is
+    left_scale * left + right_scale * right. Each side writes the input of
+    its output projection, already times its scale (applied in fp32 before
+    the value is rounded), into its half of one buffer, and ONE GEMM over
+    [left | right] with the two projections' columns side by side makes the
+    sum. At most one side keeps pages; the layer's state is the list of
+    both sides' pieces."""
+
+    def __init__(self, left: nn.Module, right: nn.Module, left_scale: float,
+                 right_scale: float):
+        super().__init__()
+        if left.kv_spec() is not None and right.kv_spec() is not None:
+            raise ValueError("only one side of a parallel mixer may keep "
+                             "pages")
+        self.left, self.right = left, right
+        self.left_scale, self.right_scale = left_scale, right_scale
+        # the right half starts on a multiple of 8 columns
+        self.split = _pad8(left.out_width)
+        wl, wr = left.w_o.data, right.w_o.data
+        pad = torch.zeros(wl.shape[0], self.split - wl.shape[1],
+                          dtype=wl.dtype, device=wl.device)
+        self.w_o = nn.Parameter(torch.cat([wl, pad, wr], 1).contiguous(),
+                                requires_grad=False)
+        left.w_o = right.w_o = None       # held once, in the fused matrix
+        self.nleft = len(self._pieces(left.state_shape()))
+
+    def kv_spec(self) -> Optional[LayerKVSpec]:
+        return self.left.kv_spec() or self.right.kv_spec()
+
+    @staticmethod
+    def _pieces(shape):
+        if shape is None:
+            return []
+        if len(shape) and isinstance(shape[0], (tuple, list)):
+            return list(shape)
+        return [shape]
+
+    def state_shape(self):
+        return (self._pieces(self.left.state_shape()) +
+                self._pieces(self.right.state_shape()))
+
+    @staticmethod
+    def _part(side, pieces):
+        kind = side.state_shape()
+        if kind is None:
+            return None
+        if len(kind) and isinstance(kind[0], (tuple, list)):
+            return tuple(pieces)
+        return pieces[0]
+
+    def forward(self, h: torch.Tensor, cache, state, meta,
+                cache_v=None) -> torch.Tensor:
+        T = h.shape[0]
+        lw, rw = self.left.out_width, self.right.out_width
+        buf = torch.empty(T, self.split + rw, dtype=h.dtype, device=h.device)
+        if self.split != lw:
+            buf[:, lw: self.split] = 0
+        n = self.nleft
+        self.left.pre_output(h, cache, self._part(self.left, state[:n]), meta,
+                             cache_v, buf[:, :lw], self.left_scale)
+        self.right.pre_output(h, cache, self._part(self.right, state[n:]),
+                              meta, cache_v, buf[:, self.split:],
+                              self.right_scale)
+        return ops.linear(buf, self.w_o)

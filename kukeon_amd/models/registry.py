@@ -37,8 +37,14 @@ def _dumovik(cfg, device, **kw):
     return DumovikModel(cfg, device=device, **kw)
 
 
+def _bezizen(cfg, device, **kw):
+    from kukeon_amd.models.bezizen import BezizenModel
+    return BezizenModel(cfg, device=device, **kw)
+
+
 # family -> constructor(cfg, device, **kw)
 FAMILIES: Dict[str, Callable] = {
+    "bezizen": _bezizen,
     "dumovik": _dumovik,
     "llama": _llama,
     "mixtral": _mixtral,
@@ -51,6 +57,7 @@ ARCHITECTURES: Dict[str, str] = {
     "Lipedra": "lipedra",
     "Rasesun": "rasesun",
     "Dumovik": "dumovik",
+    "Bezizen": "bezizen",
 }
 
 
@@ -62,6 +69,7 @@ OP_GROUPS: Dict[str, tuple] = {
     "lipedra": ("mix",),
     "rasesun": ("recur",),
     "dumovik": ("hyb",),
+    "bezizen": ("strm",),
 }
 
 
@@ -135,12 +143,35 @@ DUMOVIK_PRESETS = {
 }
 
 
+def _bezizen_preset(**kw):
+    def make():
+        from kukeon_amd.models.bezizen import bezizen_bench
+        return bezizen_bench(**kw)
+    return make
+
+
+# random-weight Bezizen stacks: three wkv layers to one parallel layer over
+# four residual streams at Llama-3-8B width, and a small one
+BEZIZEN_PRESETS = {
+    "bezizen-8b-like": _bezizen_preset(width=4096, layers=32, heads=32,
+                                       kv_heads=8, ff=14336, vocab=128256,
+                                       name="bezizen-8b-like"),
+    "tiny-bezizen": _bezizen_preset(width=128, layers=4, heads=4, kv_heads=2,
+                                    ff=256, vocab=384, window=24, experts=8,
+                                    streams=2, max_positions=512,
+                                    name="tiny-bezizen"),
+}
+
+
 def preset_names():
     return sorted(list(MODEL_PRESETS) + list(LIPEDRA_PRESETS) +
-                  list(RASESUN_PRESETS) + list(DUMOVIK_PRESETS))
+                  list(RASESUN_PRESETS) + list(DUMOVIK_PRESETS) +
+                  list(BEZIZEN_PRESETS))
 
 
 def preset(name: str):
+    if name in BEZIZEN_PRESETS:
+        return BEZIZEN_PRESETS[name]()
     if name in DUMOVIK_PRESETS:
         return DUMOVIK_PRESETS[name]()
     if name in LIPEDRA_PRESETS:
@@ -172,5 +203,9 @@ def load_checkpoint(model_dir: str, device, dtype: str = "bf16"):
     if fam == "dumovik":
         from kukeon_amd.models.dumovik import DumovikModel
         return DumovikModel.from_checkpoint(model_dir, device=device,
+                                            dtype=dtype)
+    if fam == "bezizen":
+        from kukeon_amd.models.bezizen import BezizenModel
+        return BezizenModel.from_checkpoint(model_dir, device=device,
                                             dtype=dtype)
     raise ValueError(f"family {fam} has no checkpoint loader")

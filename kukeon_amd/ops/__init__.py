@@ -122,6 +122,42 @@ def _hyb(t: torch.Tensor):
     return _C_hyb
 
 
+_C_strm = None
+_STRM_IMPORT_ERROR: Exception | None = None
+try:
+    from kukeon_amd import _C_strm  # type: ignore
+except Exception as e:  # pragma: no cover
+    _STRM_IMPORT_ERROR = e
+
+
+def strm_available() -> bool:
+    return _C_strm is not None
+
+
+def _strm(t: torch.Tensor):
+    """Kernel group of the multi-stream stacks (stream read/write with the
+    norm, token shift, linear attention with a decay per key channel,
+    windowed attention with a distance bias, group-limited routing): native
+    on a GPU tensor (an error if the module is not built), fp32 references
+    on CPU."""
+    global _C_strm, _STRM_IMPORT_ERROR
+    if not t.is_cuda:
+        return reference
+    if _C_strm is None:
+        try:
+            import importlib
+            _C_strm = importlib.import_module("kukeon_amd._C_strm")
+        except Exception as e:
+            _STRM_IMPORT_ERROR = e
+    if _C_strm is None:
+        raise RuntimeError(
+            "kukeon_amd._C_strm (gfx950 HIP extension) is not built but an "
+            "op was called on a CUDA device. Run `python -m "
+            f"kukeon_amd.ops.build strm` (import error: "
+            f"{_STRM_IMPORT_ERROR})")
+    return _C_strm
+
+
 def _shared(t: torch.Tensor, first, second):
     """A kernel that two groups compile from the same source: whichever of
     the two modules is built serves it (`first` preferred)."""
@@ -139,6 +175,25 @@ def _shared(t: torch.Tensor, first, second):
 
 
 _SHARED_CHOICE: dict = {}
+
+
+def _shared3(t: torch.Tensor, first, second, third):
+    """As _shared, for a kernel that three groups compile."""
+    if not t.is_cuda:
+        return reference
+    key = (first, second, third)
+    mod = _SHARED_CHOICE.get(key)
+    if mod is None:
+        for get in key:
+            try:
+                mod = get(t)
+                break
+            except RuntimeError as e:
+                err = e
+        if mod is None:
+            raise err
+        _SHARED_CHOICE[key] = mod
+    return mod
 
 
 def _native():
@@ -436,7 +491,7 @@ def residual_add_rmsnorm(x, a, bias, w, w_offset: float, eps: float,
 def clamp_glu(out, gate, up, bg, bu, limit: float, alpha: float = 1.702,
               up_shift: float = 1.0) -> None:
     none = torch.empty(0, dtype=torch.float32, device=out.device)
-    _shared(out, _mix, _hyb).clamp_glu(
+    _shared3(out, _mix, _hyb, _strm).clamp_glu(
         out, gate, up, bg if bg is not None else none,
         bu if bu is not None else none, limit, alpha, up_shift)
 
@@ -595,7 +650,7 @@ def table_moe(out, h, ids, table, w_up, w_down) -> None:
 
 
 def gather_rows(out, inp, row_map) -> None:
-    _shared(out, _recur, _hyb).gather_rows(out, inp, row_map)
+    _shared3(out, _recur, _hyb, _strm).gather_rows(out, inp, row_map)
 
 
 def relu_square_(x) -> None:
@@ -679,4 +734,111 @@ def router_topk(idx, wts, logits, top: int, dense_rows: int = 0) -> None:
 
 
 def combine_rows_weighted(out, inp, inv, wts) -> None:
-    _hyb(out).combine_rows_weighted(out, inp, inv, wts)
+    _shared(out, _hyb, _strm).combine_rows_weighted(out, inp, inv, wts)
+
+
+# ---- stream group ----------------------------------------------------------
+def embed_streams(xs, ids, positions, table, pos_table, scale: float) -> None:
+    """xs [T, S, W] fp32: every stream = table[id] * scale + pos_table[p]."""
+    _strm(xs).embed_streams(xs, ids, positions, table,
+                            pos_table if pos_table is not None else _e(table),
+                            scale)
+
+
+def stream_read_norm(out, xs, coef, w, eps: float) -> None:
+    """out = rmsnorm(sum_s coef[s] xs[:, s]) * w."""
+    _strm(xs).stream_read_norm(out, xs, coef, w, eps)
+
+
+def stream_write_read_norm(xs, y, mix, outc, coef, w, eps: float,
+                           out) -> None:
+    """xs[:, j] <- sum_s mix[s, j] xs[:, s] + outc[j] y in place, then the
+    next sublayer's read: out = rmsnorm(sum_j coef[j] xs[:, j]) * w."""
+    _strm(xs).stream_write_read_norm(xs, y, mix, outc, coef, w, eps, out)
+
+
+def token_shift(out, h, mu, state, positions, row_seq, cu_rows, state_slots,
+                shift_state: bool = False) -> None:
+    """out[n] = h + (row before - h) * mu[n]; the row before a portion's
+    first comes from the state slot."""
+    _strm(h).token_shift(out, h, mu, state, positions, row_seq, cu_rows,
+                         state_slots, shift_state)
+
+
+def token_shift_tail(state, h, positions, cu_rows, state_slots) -> None:
+    _strm(h).token_shift_tail(state, h, positions, cu_rows, state_slots)
+
+
+def tanh_cast(out, z) -> None:
+    _strm(out).tanh_cast(out, z)
+
+
+def decay_scan(y, q, k, v, z, zb, bonus, state, positions, cu_rows,
+               state_slots, H: int, d: int, dv: int, mode: int,
+               tau: float = 1.0, q_scale: float = 1.0) -> None:
+    _strm(q).decay_scan(y, q, k, v, z, zb,
+                        bonus if bonus is not None else _e(zb), state,
+                        positions, cu_rows, state_slots, H, d, dv, mode, tau,
+                        q_scale)
+
+
+def head_rmsnorm_gate(out, y, gate, w, H: int, eps: float, act: int,
+                      scale: float = 1.0) -> None:
+    """out (a [T, C] view) = y / rms_per_head(y) * w * act(gate) * scale;
+    act 0 = silu, 1 = sigmoid."""
+    _strm(out).head_rmsnorm_gate(out, y, gate, w, H, eps, act, scale)
+
+
+def scaled_gate(out, a, gate, act: int, scale: float = 1.0) -> None:
+    """out (a [T, C] view) = a * act(gate) * scale; act 0 = silu,
+    1 = sigmoid."""
+    _strm(out).scaled_gate(out, a, gate, act, scale)
+
+
+def conv_scale_append(q_out, k_cache, proj, q_col: int, k_col: int, cw, state,
+                      coef: float, every: int, positions, row_seq, cu_rows,
+                      state_slots, block_table,
+                      shift_state: bool = False) -> None:
+    _strm(proj).conv_scale_append(q_out, k_cache, proj, q_col, k_col, cw,
+                                  state, coef, every, positions, row_seq,
+                                  cu_rows, state_slots, block_table,
+                                  shift_state)
+
+
+def conv_pair_tail_update(state, proj, q_col: int, k_col: int, Cq: int,
+                          Ck: int, zero_bias, positions, cu_rows,
+                          state_slots) -> None:
+    """Shift a portion's last query and key inputs into the slots."""
+    _strm(proj).conv_state_update(state, proj, zero_bias, positions, cu_rows,
+                                  state_slots, q_col, k_col, 0, Cq, Ck, 0)
+
+
+def window_attention(out, q, k_cache, v_cache, slopes, positions, row_seq,
+                     block_table, H: int, scale: float, window: int) -> None:
+    """Values are the keys when v_cache is None or empty."""
+    _strm(q).window_attention(out, q, k_cache,
+                              v_cache if v_cache is not None else _e(q),
+                              slopes if slopes is not None
+                              else torch.empty(0, dtype=torch.float32,
+                                               device=q.device),
+                              positions, row_seq, block_table, H, scale,
+                              window)
+
+
+def window_tiles_supported(t: torch.Tensor, d: int, BS: int) -> bool:
+    return (t.is_cuda and t.dtype == torch.bfloat16
+            and _strm(t).window_attention_tiles_supported(d, BS))
+
+
+def window_attention_tiles(out, q, k_cache, slopes, block_table, seq_lens,
+                           q_starts, qb_seq, qb_start, scale: float,
+                           window: int) -> None:
+    _strm(q).window_attention_tiles(out, q, k_cache, slopes, block_table,
+                                    seq_lens, q_starts, qb_seq, qb_start,
+                                    scale, window)
+
+
+def router_select(idx, wts, logits, top: int, groups: int, keep: int,
+                  scale: float, dense_rows: int = 0) -> None:
+    _strm(logits).router_select(idx, wts, logits, top, groups, keep, scale,
+                                dense_rows)

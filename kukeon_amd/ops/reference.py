@@ -727,3 +727,240 @@ def combine_rows_weighted(out, inp, inv, wts) -> None:
     """out[t] = sum over k of wts[t, k] * inp[inv[t, k]]."""
     out.copy_((inp[inv.long()].float() * wts[:, :, None]).sum(1).to(
         out.dtype))
+
+
+# ---------------------------------------------------------------------------
+# stream group (several residual streams with learned read/write weights,
+# token shift, linear attention with a decay per key channel, windowed
+# attention with a distance bias, group-limited routing)
+# ---------------------------------------------------------------------------
+
+def embed_streams(xs, ids, positions, table, pos_table, scale: float) -> None:
+    """xs[r, s] = table[ids[r]] * scale + pos_table[positions[r]] for every
+    stream s (fp32); an inactive row (position < 0) gets zeros."""
+    p = positions.long()
+    live = (p >= 0)
+    x = table[ids.long()].float() * scale
+    if pos_table is not None and pos_table.numel():
+        x = x + pos_table[p.clamp_min(0)].float()
+    x = x * live[:, None]
+    xs.copy_(x[:, None, :].expand_as(xs))
+
+
+def stream_read_norm(out, xs, coef, w, eps: float) -> None:
+    """out = rmsnorm(sum_s coef[s] xs[:, s]) * w."""
+    u = (xs * coef[None, :, None]).sum(1)
+    out.copy_((_unit_rms(u, eps) * w).to(out.dtype))
+
+
+def stream_write_read_norm(xs, y, mix, outc, coef, w, eps: float,
+                           out) -> None:
+    """xs[:, j] <- sum_s mix[s, j] xs[:, s] + outc[j] y (all streams from the
+    old ones, in place), then out = rmsnorm(sum_j coef[j] xs[:, j]) * w."""
+    new = torch.einsum("sj,tsw->tjw", mix, xs) + \
+        outc[None, :, None] * y.float()[:, None, :]
+    xs.copy_(new)
+    stream_read_norm(out, xs, coef, w, eps)
+
+
+def token_shift(out, h, mu, state, positions, row_seq, cu_rows, state_slots,
+                shift_state: bool = False) -> None:
+    """out[n, r] = h[r] + (prev[r] - h[r]) * mu[n], prev being the row before
+    in the same sequence: the portion's own, or the state slot's for its
+    first row (zeros at position 0). With `shift_state` (one row per
+    sequence) the slot takes h[r] in the same call."""
+    nseq = cu_rows.numel() - 1
+    hf = h.float()
+    for s in range(nseq):
+        r0, r1 = int(cu_rows[s]), int(cu_rows[s + 1])
+        if r1 <= r0 or int(positions[r0]) < 0:
+            continue
+        slot = int(state_slots[s])
+        first = state[slot].clone() if int(positions[r0]) > 0 else \
+            torch.zeros_like(state[slot])
+        prev = torch.cat([first[None], hf[r0:r1 - 1]], 0)
+        cur = hf[r0:r1]
+        out[:, r0:r1] = (cur[None] + (prev - cur)[None] * mu[:, None, :]).to(
+            out.dtype)
+        if shift_state:
+            state[slot] = hf[r1 - 1]
+
+
+def token_shift_tail(state, h, positions, cu_rows, state_slots) -> None:
+    """state[slot of s] = the last row of sequence s's portion."""
+    nseq = cu_rows.numel() - 1
+    for s in range(nseq):
+        r0, r1 = int(cu_rows[s]), int(cu_rows[s + 1])
+        if r1 <= r0 or int(positions[r0]) < 0:
+            continue
+        state[int(state_slots[s])] = h[r1 - 1].float()
+
+
+def tanh_cast(out, z) -> None:
+    out.copy_(torch.tanh(z.float()).to(out.dtype))
+
+
+def decay_scan(y, q, k, v, z, zb, bonus, state, positions, cu_rows,
+               state_slots, H: int, d: int, dv: int, mode: int, tau: float,
+               q_scale: float) -> None:
+    """Linear attention with a decay per key channel, token after token.
+    Decay a_t = exp(-exp(z_t + zb)) (mode 0) or sigmoid(z_t + zb)^(1/tau)
+    (mode 1), fp32. Mode 0 reads before it writes and gives the current
+    token a bonus: y_t = (S + diag(bonus) k_t v_t^T)^T q_t, then
+    S = diag(a_t) S + k_t v_t^T. Mode 1: S = diag(a_t) S + k_t v_t^T, then
+    y_t = S^T (q_scale q_t). state [slots, H, dv, d] holds S^T (zeros at
+    position 0); y [T, H*dv] fp32; q, k [T, H*d], v [T, H*dv] views."""
+    nseq = cu_rows.numel() - 1
+    for s in range(nseq):
+        r0, r1 = int(cu_rows[s]), int(cu_rows[s + 1])
+        if r1 <= r0:
+            continue
+        if int(positions[r0]) < 0:
+            y[r0:r1] = 0
+            continue
+        slot = int(state_slots[s])
+        S = state[slot].transpose(1, 2).clone()              # [H, d, dv]
+        if int(positions[r0]) == 0:
+            S.zero_()
+        for r in range(r0, r1):
+            qq = q[r].float().view(H, d) * q_scale
+            kk = k[r].float().view(H, d)
+            vv = v[r].float().view(H, dv)
+            zz = (z[r].float() + zb).view(H, d)
+            kv = kk[:, :, None] * vv[:, None, :]
+            if mode == 0:
+                a = torch.exp(-torch.exp(zz))
+                y[r] = ((S + bonus.view(H, d)[:, :, None] * kv) *
+                        qq[:, :, None]).sum(1).reshape(H * dv)
+                S = a[:, :, None] * S + kv
+            else:
+                a = torch.exp(torch.nn.functional.logsigmoid(zz) / tau)
+                S = a[:, :, None] * S + kv
+                y[r] = (S * qq[:, :, None]).sum(1).reshape(H * dv)
+        state[slot] = S.transpose(1, 2)
+
+
+def _gate_act(gate, act: int):
+    g = gate.float()
+    return g * torch.sigmoid(g) if act == 0 else torch.sigmoid(g)
+
+
+def head_rmsnorm_gate(out, y, gate, w, H: int, eps: float, act: int,
+                      scale: float = 1.0) -> None:
+    """out = y / rms_per_head(y) * w * act(gate) * scale: act 0 = silu,
+    1 = sigmoid; the row is cut into H heads, each divided by its own root
+    mean square."""
+    T, C = y.shape
+    n = _unit_rms(y.float().view(T, H, C // H), eps).view(T, C) * w
+    out.copy_((n * _gate_act(gate, act) * scale).to(out.dtype))
+
+
+def scaled_gate(out, a, gate, act: int, scale: float = 1.0) -> None:
+    """out = a * act(gate) * scale."""
+    out.copy_((a.float() * _gate_act(gate, act) * scale).to(out.dtype))
+
+
+def conv_scale_append(q_out, k_cache, proj, q_col: int, k_col: int, cw, state,
+                      coef: float, every: int, positions, row_seq, cu_rows,
+                      state_slots, block_table,
+                      shift_state: bool = False) -> None:
+    """Short causal convolution (no bias, no activation) over the query and
+    the key columns of a projection, carried taps in `state`
+    [slots, taps-1, Cq+Ck]. The queries are scaled by
+    1 + coef ln(floor((p + 1) / every) + 1) and go to q_out [T, Cq]; the
+    keys go to the row's page, k_cache [blocks, G, BS, d]."""
+    taps, C = cw.shape
+    Cq = q_out.shape[1]
+    Ck = C - Cq
+    back = taps - 1
+    G, BS = k_cache.shape[1], k_cache.shape[2]
+    cols = _conv_cols(q_col, k_col, 0, Cq, Ck, 0)
+    nseq = cu_rows.numel() - 1
+    for s in range(nseq):
+        r0, r1 = int(cu_rows[s]), int(cu_rows[s + 1])
+        if r1 <= r0 or int(positions[r0]) < 0:
+            continue
+        n = r1 - r0
+        p0 = int(positions[r0])
+        u = proj[r0:r1][:, cols].float()
+        slot = int(state_slots[s])
+        hist = state[slot].clone() if back else u[:0]
+        for j in range(back):
+            if p0 - back + j < 0:
+                hist[j] = 0
+        full = torch.cat([hist, u], 0)
+        yv = torch.zeros(n, C)
+        for j in range(taps):
+            yv = yv + cw[j] * full[j: j + n]
+        pp = torch.arange(p0, p0 + n)
+        temp = torch.ones(n)
+        if every > 0:
+            temp = 1.0 + coef * torch.log(
+                torch.div(pp + 1, every, rounding_mode="floor").float() + 1.0)
+        q_out[r0:r1] = (yv[:, :Cq] * temp[:, None]).to(q_out.dtype)
+        kk = yv[:, Cq:].reshape(n, G, -1).to(k_cache.dtype)
+        for i in range(n):
+            p = p0 + i
+            blk = int(block_table[s, p // BS])
+            k_cache[blk, :, p % BS] = kk[i]
+        if shift_state and back:
+            state[slot] = full[-back:]
+
+
+def window_attention(out, q, k_cache, v_cache, slopes, positions, row_seq,
+                     block_table, H: int, scale: float, window: int) -> None:
+    """Grouped-query softmax attention of row r (position p) over the keys
+    max(0, p - window + 1) .. p (all of 0 .. p when window is 0), with
+    slopes[h] (p - j) taken off head h's scores. Without a value cache
+    (None or empty) the values are the keys."""
+    G, BS, d = k_cache.shape[1], k_cache.shape[2], k_cache.shape[3]
+    own_v = v_cache is not None and v_cache.numel() > 0
+    dv = v_cache.shape[3] if own_v else d
+    for r in range(q.shape[0]):
+        p = int(positions[r])
+        if p < 0:
+            out[r] = 0
+            continue
+        s = int(row_seq[r])
+        lo = max(0, p - window + 1) if window > 0 else 0
+        js = torch.arange(lo, p + 1)
+        blk = block_table[s, (js // BS).long()].long()
+        k = k_cache[blk, :, (js % BS).long()].float()         # [n, G, d]
+        v = v_cache[blk, :, (js % BS).long()].float() if own_v else k
+        qr = q[r].float().view(H, d)
+        for h in range(H):
+            g = h // (H // G)
+            sc = (k[:, g] @ qr[h]) * scale
+            if slopes is not None and slopes.numel():
+                sc = sc - slopes[h] * (p - js).float()
+            out[r, h * dv:(h + 1) * dv] = (torch.softmax(sc, -1) @
+                                           v[:, g]).to(out.dtype)
+
+
+def router_select(idx, wts, logits, top: int, groups: int, keep: int,
+                  scale: float, dense_rows: int = 0) -> None:
+    """Scores = softmax over all logits. With groups > 0 the experts form
+    `groups` equal runs of neighbours, a run's score is its largest, and
+    only the `keep` best runs can be chosen (ties: the lower index). The
+    `top` best allowed experts get their scores divided by the scores' sum
+    (+ 1e-20), times scale. With dense_rows = T the index written is
+    expert * T + row. idx and wts may have more than `top` columns; the
+    others are left alone."""
+    T, E = logits.shape
+    s = torch.softmax(logits.float(), -1)
+    allowed = s.clone()
+    if groups > 0:
+        best = s.view(T, groups, E // groups).max(-1).values
+        kept = torch.sort(best, dim=-1, descending=True,
+                          stable=True).indices[:, :keep]
+        mask = torch.zeros(T, groups, dtype=torch.bool)
+        mask.scatter_(1, kept, True)
+        allowed = torch.where(mask.repeat_interleave(E // groups, 1), s,
+                              torch.full_like(s, -1.0))
+    ix = torch.sort(allowed, dim=-1, descending=True,
+                    stable=True).indices[:, :top]
+    w = s.gather(1, ix)
+    wts[:, :top] = w / (w.sum(-1, keepdim=True) + 1e-20) * scale
+    if dense_rows:
+        ix = ix * dense_rows + torch.arange(T)[:, None]
+    idx[:, :top] = ix.to(idx.dtype)

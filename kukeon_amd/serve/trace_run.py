@@ -80,6 +80,8 @@ def main(argv=None) -> int:
         dtype="fp32" if args.dtype == "float32" else "bf16")
     max_len = nblocks * bs
     model.set_max_position(max_len)
+    # a model with a position table bounds the longest sequence itself
+    max_len = min(max_len, getattr(model, "max_position", max_len))
     ecfg = EngineConfig(block_size=bs, max_model_len=max_len,
                         max_sessions=args.slots, state_slots=args.slots,
                         num_kv_blocks=nblocks, use_graphs=False)
