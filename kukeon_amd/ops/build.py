@@ -64,6 +64,23 @@ HYB_SOURCES = [
     "bindings_hyb.cpp",
 ]
 
+#   strm -> kukeon_amd/_C_strm.so (several residual streams, token shift,
+#                                  linear attention with a token-dependent
+#                                  decay, windowed attention over key-only
+#                                  pages, group-limited routing)
+STRM_SOURCES = [
+    "stream_mix.hip",
+    "decay_scan.hip",
+    "window_attn.hip",
+    "short_conv.hip",
+    "chunk_attn.hip",
+    "prefill_attn.hip",
+    "routed_moe.hip",
+    "glu_clamp.hip",
+    "table_moe.hip",
+    "bindings_strm.cpp",
+]
+
 SOURCES = [
     "rmsnorm.hip",
     "activation.hip",
@@ -96,6 +113,7 @@ GROUPS = {
     "mix": ("_C_mix", MIX_SOURCES),
     "recur": ("_C_recur", RECUR_SOURCES),
     "hyb": ("_C_hyb", HYB_SOURCES),
+    "strm": ("_C_strm", STRM_SOURCES),
 }
 
 

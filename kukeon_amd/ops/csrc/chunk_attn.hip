@@ -1,7 +1,10 @@
 // Grouped-query attention whose scores carry no positions: queries and keys
 // are RMS-normed over their WHOLE projection row, scores are scaled and may
 // be capped (cap tanh(score / cap)), and a query at position p sees the keys
-// lo .. p, lo being the first position of p's chunk (0 without chunks).
+// lo .. p, lo being the first position of p's chunk (0 without chunks). The
+// same kernel serves a sliding window (lo = p - window + 1), a distance bias
+// slope_h (p - j) taken off head h's scores, and caches without value rows,
+// where the values are the keys (window_attention).
 //
 // qk_norm_append   norms q (and k) of every row, writes q to a dense buffer
 //                  and k, v to the row's page.
@@ -209,7 +212,7 @@ __global__ __launch_bounds__(1024) void chunk_attention_kernel(
     const T* __restrict__ vc, const int* __restrict__ positions,
     const int* __restrict__ row_seq, const int* __restrict__ block_table,
     int max_blocks, int H, int G, int d, int dq, int dv, int BS, float scale,
-    float cap, int chunk) {
+    float cap, int chunk, int window, const float* __restrict__ slopes) {
   extern __shared__ float sm[];
   const int tid = threadIdx.x;
   const int wave = tid / WAVE;
@@ -249,7 +252,12 @@ __global__ __launch_bounds__(1024) void chunk_attention_kernel(
   __syncthreads();
 
   const int s = row_seq[r];
-  const int lo = chunk > 0 ? (p / chunk) * chunk : 0;
+  int lo = chunk > 0 ? (p / chunk) * chunk : 0;
+  if (window > 0) lo = max(lo, p - window + 1);
+  float slope[CA_HB];
+#pragma unroll
+  for (int hb = 0; hb < CA_HB; ++hb)
+    slope[hb] = (slopes && hb < nh) ? slopes[h0 + hb] : 0.f;
   float m[CA_HB], l[CA_HB], acc[CA_HB][8];
 #pragma unroll
   for (int hb = 0; hb < CA_HB; ++hb) {
@@ -298,6 +306,7 @@ __global__ __launch_bounds__(1024) void chunk_attention_kernel(
       for (int hb = 0; hb < CA_HB; ++hb) {
         sc[hb] = dot[hb] * scale;
         if (cap > 0.f) sc[hb] = cap * tanhf(sc[hb] / cap);
+        sc[hb] -= slope[hb] * (float)(p - j);
       }
     }
 #pragma unroll
@@ -399,12 +408,22 @@ __global__ __launch_bounds__(1024) void chunk_attention_kernel(
   }
 }
 
-// out [T, H*dv], q [T, H*d] contiguous; caches as in qk_norm_append.
-void chunk_attention(torch::Tensor out, torch::Tensor q, torch::Tensor k_cache,
-                     torch::Tensor v_cache, torch::Tensor positions,
-                     torch::Tensor row_seq, torch::Tensor block_table,
-                     int64_t H, double scale, double softcap, int64_t chunk) {
+// out [T, H*dv], q [T, H*d] contiguous; caches as in qk_norm_append. An
+// empty v_cache means that the values are the keys; slopes [H] fp32 or empty.
+static void masked_attention(torch::Tensor out, torch::Tensor q,
+                             torch::Tensor k_cache, torch::Tensor v_cache,
+                             torch::Tensor slopes, torch::Tensor positions,
+                             torch::Tensor row_seq, torch::Tensor block_table,
+                             int64_t H, double scale, double softcap,
+                             int64_t chunk, int64_t window) {
   check_act(q, "q");
+  if (v_cache.numel() == 0) v_cache = k_cache;
+  const bool biased = slopes.numel() > 0;
+  if (biased) {
+    check_f32(slopes, "slopes");
+    TORCH_CHECK(slopes.numel() == H);
+  }
+  TORCH_CHECK(window >= 0);
   check_i32(positions, "positions"); check_i32(row_seq, "row_seq");
   check_i32(block_table, "block_table");
   TORCH_CHECK(k_cache.dim() == 4 && k_cache.is_contiguous() &&
@@ -449,7 +468,8 @@ void chunk_attention(torch::Tensor out, torch::Tensor q, torch::Tensor k_cache,
         reinterpret_cast<const T*>(v_cache.data_ptr()),                    \
         positions.data_ptr<int>(), row_seq.data_ptr<int>(),                \
         block_table.data_ptr<int>(), (int)block_table.size(1), (int)H, G,  \
-        d, dq, dv, BS, (float)scale, (float)softcap, (int)chunk
+        d, dq, dv, BS, (float)scale, (float)softcap, (int)chunk,           \
+        (int)window, biased ? slopes.data_ptr<float>() : nullptr
   KK_DISPATCH_ACT(q, {
     if (vec) {
       auto kern = chunk_attention_kernel<T, true>;
@@ -477,6 +497,27 @@ void chunk_attention(torch::Tensor out, torch::Tensor q, torch::Tensor k_cache,
   });
 #undef KK_ARGS
   HIP_CHECK_KERNEL();
+}
+
+void chunk_attention(torch::Tensor out, torch::Tensor q, torch::Tensor k_cache,
+                     torch::Tensor v_cache, torch::Tensor positions,
+                     torch::Tensor row_seq, torch::Tensor block_table,
+                     int64_t H, double scale, double softcap, int64_t chunk) {
+  masked_attention(out, q, k_cache, v_cache,
+                   torch::empty({0}, positions.options().dtype(torch::kFloat32)),
+                   positions, row_seq, block_table, H, scale, softcap, chunk,
+                   0);
+}
+
+// Sliding-window attention with a distance bias; an empty v_cache makes the
+// keys the values.
+void window_attention(torch::Tensor out, torch::Tensor q, torch::Tensor k_cache,
+                      torch::Tensor v_cache, torch::Tensor slopes,
+                      torch::Tensor positions, torch::Tensor row_seq,
+                      torch::Tensor block_table, int64_t H, double scale,
+                      int64_t window) {
+  masked_attention(out, q, k_cache, v_cache, slopes, positions, row_seq,
+                   block_table, H, scale, 0.0, 0, window);
 }
 
 }  // namespace kukeon

@@ -126,7 +126,10 @@ DEV_INLINE unsigned int cvt_pk_bf16(float lo, float hi) {
 // EXT adds what chunk-local attention with capped scores needs: keys start at
 // the first position of the query's chunk, scores pass cap * tanh(s / cap),
 // and the softmax weights enter the PV product as hi + lo (two bf16 terms)
-// so that they keep fp32-grade accuracy.
+// so that they keep fp32-grade accuracy. EXT also serves a sliding window
+// (keys from q - window + 1 on) and a distance bias slope_h (q - k) taken off
+// head h's scores; with the key cache passed as the value cache too, the
+// values are the keys.
 template <int BS, bool FP8, bool EXT>
 __global__ __launch_bounds__(256, 1) void prefill_attn_kernel(
     unsigned short* __restrict__ out,       // [T, Hq*D]
@@ -139,7 +142,8 @@ __global__ __launch_bounds__(256, 1) void prefill_attn_kernel(
     const int* __restrict__ qb_seq,         // [nqb]
     const int* __restrict__ qb_start,       // [nqb] local q offset
     long q_stride, long q_offset, int Hq, int Hk, int max_blocks,
-    int out_stride, float scale, float cap, int chunk) {
+    int out_stride, float scale, float cap, int chunk, int window,
+    const float* __restrict__ slopes) {
   constexpr int D = 128;
   constexpr int KVT = 32;
   // 16-B aligned: staged via uint4 stores (guide G17)
@@ -167,9 +171,13 @@ __global__ __launch_bounds__(256, 1) void prefill_attn_kernel(
   // absolute position of this lane's q column (clamped for padding rows)
   const int q_abs = abs_start + qb0 + min(qcol, qn - 1);
   // first key this lane's query sees, and the first any row of the tile sees
-  const int q_lo = (EXT && chunk > 0) ? (q_abs / chunk) * chunk : 0;
-  const int tile_lo =
-      (EXT && chunk > 0) ? ((abs_start + qb0) / chunk) * chunk : 0;
+  int q_lo = (EXT && chunk > 0) ? (q_abs / chunk) * chunk : 0;
+  int tile_lo = (EXT && chunk > 0) ? ((abs_start + qb0) / chunk) * chunk : 0;
+  if (EXT && window > 0) {
+    q_lo = max(q_lo, q_abs - window + 1);
+    tile_lo = max(tile_lo, abs_start + qb0 - window + 1);
+  }
+  const float slope = (EXT && slopes) ? slopes[head] : 0.f;
 
   // ---- load Q fragments (B-operand: col=q, k=d chunks) ----
   unsigned int qfrag[8][4];
@@ -291,6 +299,7 @@ __global__ __launch_bounds__(256, 1) void prefill_attn_kernel(
                          (!EXT || kvpos >= q_lo);
       float sc = sacc[r] * scale;
       if (EXT && cap > 0.f) sc = cap * tanhf(sc / cap);
+      if (EXT) sc -= slope * (float)(q_abs - kvpos);
       sv[r] = valid ? sc : -INFINITY;
       tmax = fmaxf(tmax, sv[r]);
     }
@@ -417,7 +426,7 @@ void prefill_attention(torch::Tensor out, torch::Tensor q,
       seq_lens.data_ptr<int>(), q_starts.data_ptr<int>(),                    \
       qb_seq.data_ptr<int>(), qb_start.data_ptr<int>(), q.stride(0),         \
       q_offset, Hq, Hk, (int)block_table.size(1), (int)out.stride(0),        \
-      (float)scale, 0.f, 0)
+      (float)scale, 0.f, 0, 0, nullptr)
   if (fp8) { PF_LAUNCH(true); } else { PF_LAUNCH(false); }
 #undef PF_LAUNCH
   HIP_CHECK_KERNEL();
@@ -470,7 +479,60 @@ void chunk_attention_tiles(torch::Tensor out, torch::Tensor q,
       seq_lens.data_ptr<int>(), q_starts.data_ptr<int>(),
       qb_seq.data_ptr<int>(), qb_start.data_ptr<int>(), q.stride(0), 0L, Hq,
       Hk, (int)block_table.size(1), (int)out.stride(0), (float)scale,
-      (float)softcap, (int)chunk);
+      (float)softcap, (int)chunk, 0, nullptr);
+  HIP_CHECK_KERNEL();
+}
+
+// sizes the tile kernel serves for windowed attention over key-only pages
+bool window_attention_tiles_supported(int64_t d, int64_t BS) {
+  return d == 128 && BS == 16;
+}
+
+// Prompt portions of sliding-window attention whose values are its keys, on
+// the matrix cores (bf16, heads of 128, pages of 16): out, q [T, H*128]
+// contiguous, k_cache [blocks, G, 16, 128], slopes [H] fp32 or empty; the
+// row maps are the ones of prefill_attention.
+void window_attention_tiles(torch::Tensor out, torch::Tensor q,
+                            torch::Tensor k_cache, torch::Tensor slopes,
+                            torch::Tensor block_table, torch::Tensor seq_lens,
+                            torch::Tensor q_starts, torch::Tensor qb_seq,
+                            torch::Tensor qb_start, double scale,
+                            int64_t window) {
+  TORCH_CHECK(k_cache.dim() == 4 && k_cache.is_contiguous());
+  const int Hk = (int)k_cache.size(1);
+  TORCH_CHECK(window_attention_tiles_supported(k_cache.size(3),
+                                               k_cache.size(2)));
+  TORCH_CHECK(q.scalar_type() == torch::kBFloat16 &&
+              out.scalar_type() == torch::kBFloat16 &&
+              k_cache.scalar_type() == torch::kBFloat16);
+  TORCH_CHECK(q.dim() == 2 && q.is_contiguous() && out.dim() == 2 &&
+              out.is_contiguous() && out.size(0) == q.size(0) &&
+              out.size(1) == q.size(1) && q.size(1) % 128 == 0);
+  const int Hq = (int)(q.size(1) / 128);
+  TORCH_CHECK(Hq % Hk == 0 && window >= 0);
+  const bool biased = slopes.numel() > 0;
+  if (biased)
+    TORCH_CHECK(slopes.is_cuda() && slopes.scalar_type() == torch::kFloat32 &&
+                slopes.is_contiguous() && slopes.numel() == Hq);
+  TORCH_CHECK(q_starts.dim() == 2 && q_starts.size(1) == 2);
+  TORCH_CHECK(qb_seq.scalar_type() == torch::kInt32 &&
+              qb_start.scalar_type() == torch::kInt32 &&
+              seq_lens.scalar_type() == torch::kInt32 &&
+              block_table.scalar_type() == torch::kInt32 &&
+              q_starts.scalar_type() == torch::kInt32);
+  const int nqb = (int)qb_seq.size(0);
+  if (nqb == 0) return;
+  const int G = Hq / Hk;
+  auto stream = c10::hip::getCurrentHIPStream().stream();
+  dim3 grid(nqb, Hk, (G + 3) / 4);
+  prefill_attn_kernel<16, false, true><<<grid, 256, 0, stream>>>(
+      reinterpret_cast<unsigned short*>(out.data_ptr()),
+      reinterpret_cast<const unsigned short*>(q.data_ptr()),
+      k_cache.data_ptr(), k_cache.data_ptr(), block_table.data_ptr<int>(),
+      seq_lens.data_ptr<int>(), q_starts.data_ptr<int>(),
+      qb_seq.data_ptr<int>(), qb_start.data_ptr<int>(), q.stride(0), 0L, Hq,
+      Hk, (int)block_table.size(1), (int)out.stride(0), (float)scale, 0.f, 0,
+      (int)window, biased ? slopes.data_ptr<float>() : nullptr);
   HIP_CHECK_KERNEL();
 }
 
