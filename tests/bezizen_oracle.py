@@ -28,8 +28,10 @@ def lin(x, w):
 # ---- embedding, streams, output ---------------------------------------------
 def embed(tokens, t, cfg):
     ids = torch.as_tensor(tokens, dtype=torch.long)
-    x = t["embed"][ids] * float(cfg["embedding"]["scale"])
-    return x + t["pos"][: len(tokens)]
+    x = t["embed"][ids] * float((cfg.get("embedding") or {}).get("scale", 1))
+    if "pos" in t:
+        x = x + t["pos"][: len(tokens)]
+    return x
 
 
 def streams_read(xs, coef):
@@ -47,7 +49,7 @@ def streams_write(xs, y, mix, out):
 def logits(x, t, cfg):
     eps = float(cfg["norm"]["eps"])
     return lin(unit_rms(x, eps) * t["final.norm"], t["head"]) * \
-        float(cfg["logit_scale"])
+        float(cfg.get("logit_scale", 1.0))
 
 
 # ---- time mixing with a data-dependent decay and a bonus --------------------
