@@ -251,8 +251,10 @@ def check(got, want, dtype, what=""):
     """fp32: every row within the tolerance. bf16: rounding can flip a close
     call of a router for a single token, which moves that row (and, through
     the carried state, some after it) by much more than rounding does
-    elsewhere, so one row in ten (at least one) may be off, though never as
-    far as a wrong mechanism puts it."""
+    elsewhere, so one row in ten (at least one) may be off. With groups a
+    flip can exchange ALL experts of a token, in the last layer nearly the
+    whole row, so such a row is only held below the distance of unrelated
+    rows; a wrong mechanism shows in every row."""
     e = row_errors(got, want)
     if dtype == "fp32":
         assert float(e.max()) <= tol(dtype), \
@@ -260,7 +262,7 @@ def check(got, want, dtype, what=""):
         return
     allowed = max(1, e.numel() // 10)
     over = int((e > tol(dtype)).sum())
-    assert over <= allowed and float(e.max()) <= 0.5, \
+    assert over <= allowed and float(e.max()) <= 1.0, \
         f"{what}: {over} rows over {tol(dtype)}, worst {float(e.max()):.3g}"
 
 
