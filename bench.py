@@ -16,6 +16,7 @@ import argparse
 import json
 import os
 import statistics
+import sys
 import time
 
 import torch
@@ -30,8 +31,8 @@ COMPARE_SIZES = {
 
 
 def compare_families(args) -> None:
-    """Prefill and decode tokens/s of Lipedra, Rasesun or Dumovik and of
-    Llama (or another family) through the same engine at equal sizes: same
+    """Prefill and decode tokens/s of Lipedra, Rasesun, Dumovik or Bezizen
+    and of Llama (or another family) through the same engine at equal sizes: same
     width, head counts,
     feed-forward size, layer count and vocabulary (Llama head_dim 128;
     Lipedra two score maps of 64 and value rows of 128 — equal cache bytes
@@ -40,12 +41,16 @@ def compare_families(args) -> None:
     16 table-routed experts, two active; Dumovik periods of chunk-local
     attention over 8192-token chunks, two linear-attention layers and latent
     attention, every second feed-forward a mixture of 16 routed experts, two
-    active)."""
+    active; Bezizen four residual streams, three wkv layers to one parallel
+    layer of windowed attention over 1024 tokens beside a gated linear
+    attention, a shared expert everywhere and every second feed-forward a
+    mixture of 16 routed experts, two active)."""
     from kukeon_amd.engine.config import (EngineConfig, ModelConfig,
                                           SamplingParams)
     from kukeon_amd.engine.engine import LLMEngine
     from kukeon_amd.engine.kv_cache import SequenceKV
     from kukeon_amd.models import registry
+    from kukeon_amd.models.bezizen import bezizen_bench
     from kukeon_amd.models.dumovik import dumovik_bench
     from kukeon_amd.models.lipedra import lipedra_bench
     from kukeon_amd.models.rasesun import rasesun_bench
@@ -72,6 +77,13 @@ def compare_families(args) -> None:
                                     window=1024 if on_gpu else 16,
                                     experts=16 if on_gpu else 4,
                                     name=f"rasesun-{size}")
+            elif fam == "bezizen":
+                cfg = bezizen_bench(width=W, layers=nl, heads=hq,
+                                    kv_heads=hk, ff=ff, vocab=vocab,
+                                    window=1024 if on_gpu else 16,
+                                    experts=16 if on_gpu else 4,
+                                    max_positions=2048,
+                                    name=f"bezizen-{size}")
             elif fam == "dumovik":
                 cfg = dumovik_bench(width=W, layers=nl, heads=hq,
                                     kv_heads=hk, ff=ff, vocab=vocab,
@@ -83,6 +95,8 @@ def compare_families(args) -> None:
                                     kv_heads=hk, dim=64, vdim=128, ff=ff,
                                     vocab=vocab, share_every=0,
                                     name=f"lipedra-{size}")
+            print(f"[compare] {size} {fam}: building", file=sys.stderr,
+                  flush=True)
             model = registry.build_model(cfg, device)
             ecfg = EngineConfig(max_model_len=2048, max_sessions=nseq,
                                 num_kv_blocks=nseq * 80 + 64,
@@ -105,6 +119,8 @@ def compare_families(args) -> None:
                 for kv in kvs:
                     engine.add_request(kv, torch.randint(
                         0, vocab, (plen,), generator=gen).tolist(), sp)
+                print(f"[compare] {size} {fam}: round {rnd}", file=sys.stderr,
+                      flush=True)
                 sync()
                 t0 = time.perf_counter()
                 while engine.waiting:
@@ -161,11 +177,11 @@ def main() -> None:
                          "decode throughput of the Lipedra family beside "
                          "Llama at equal layer sizes (random weights)")
     ap.add_argument("--compare-family", default="lipedra",
-                    choices=["lipedra", "rasesun", "dumovik"],
+                    choices=["lipedra", "rasesun", "dumovik", "bezizen"],
                     help="with --compare-families: the family that runs "
                          "beside Llama")
     ap.add_argument("--compare-against", default="llama",
-                    choices=["llama", "lipedra", "rasesun"],
+                    choices=["llama", "lipedra", "rasesun", "dumovik"],
                     help="with --compare-families: the family it runs "
                          "beside (default Llama)")
     ap.add_argument("--compare-sizes", default="2k,4k,8k",

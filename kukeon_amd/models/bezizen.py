@@ -147,12 +147,15 @@ def bezizen_bench(width=4096, layers=8, heads=32, kv_heads=8, ff=14336,
     """A layer stack at real-model sizes (random weights) for throughput
     runs: three wkv layers (heads of 128) to one parallel layer (windowed
     attention with heads of 128 beside a gated linear attention over a
-    quarter of the heads); every second feed-forward is absent so that the
-    routed layers carry the dense layer's active width."""
+    quarter of the heads). Every feed-forward has `ff` active rows: a
+    shared expert of a quarter of them plus `top` routed experts; in every
+    second layer the routed experts are 16 (in 4 groups, the best 2 kept),
+    in the others there are only `top` of them, all chosen (a dense layer in
+    effect, on the same kernels)."""
     ls = []
     hd = 128 if width >= 1024 else 32
     for i in range(layers):
-        if i % 4 == 3:
+        if i % 4 == 3 or (layers < 4 and i == layers - 1):
             kind = "parallel"
             mix = ParallelCfg(
                 WindowAttnCfg(heads=heads, kv_heads=kv_heads, dim=hd,
@@ -164,10 +167,11 @@ def bezizen_bench(width=4096, layers=8, heads=32, kv_heads=8, ff=14336,
             kind = "wkv"
             mix = WkvCfg(heads=max(1, width // hd), dim=hd)
         sh = max(8, ff // 4 // 8 * 8)
+        ne = experts if i % 2 else top
+        grouped = ne % 4 == 0 and ne >= 8 and top <= ne // 2
         mlp = FFCfg("moe", max(8, (ff - sh) // top // 8 * 8),
-                    experts=experts, top=top, act="silu", score="all",
-                    groups=4 if experts % 4 == 0 and experts >= 8 else 0,
-                    keep=2 if experts % 4 == 0 and experts >= 8 else 0,
+                    experts=ne, top=top, act="silu", score="all",
+                    groups=4 if grouped else 0, keep=2 if grouped else 0,
                     route_scale=1.0, shared_ff=sh)
         ls.append(BezizenLayerCfg(kind, mix, mlp))
     return BezizenConfig(name=name, width=width, vocab_size=vocab,

@@ -36,6 +36,15 @@ class FFCfg:
     shared_ff: int = 0       # hidden size of an always-on expert (0: none)
 
 
+def pad_rows(w: torch.Tensor, multiple: int) -> torch.Tensor:
+    """w with zero rows appended up to a multiple of `multiple` rows."""
+    n = -w.shape[0] % multiple
+    if not n:
+        return w
+    return torch.cat([w, torch.zeros(n, w.shape[1], dtype=w.dtype,
+                                     device=w.device)], 0).contiguous()
+
+
 def _softplus(x: float) -> float:
     return x if x > 30 else math.log1p(math.exp(x))
 
@@ -249,6 +258,10 @@ class RoutedMoE(nn.Module):
         # in the activation format: products of two bf16 numbers are exact
         # in fp32, so the fp32-output GEMM over bf16 rows IS the fp32 router
         self.w_router = t[p + "router"].to(**dev).contiguous()
+        if f.score == "all" and f.experts % 16:
+            # the score product is made 16 columns wide at least (zero rows
+            # below the experts'); the router reads the first `experts`
+            self.w_router = pad_rows(self.w_router, 16)
 
     @staticmethod
     def tensor_shapes(f: FFCfg, width: int, vocab: int) -> Dict[str, tuple]:
@@ -296,7 +309,7 @@ class RoutedMoE(nn.Module):
                 meta=None) -> torch.Tensor:
         f = self.f
         T, W = h.shape
-        logits = ops.linear_f32(h, self.w_router)
+        logits = ops.linear_f32(h, self.w_router)[:, :f.experts]
         # with a shared expert the fold takes one more row per token
         cols = f.top + (1 if self.shared is not None else 0)
         idx = torch.empty(T, cols, dtype=torch.int32, device=h.device)
@@ -314,11 +327,14 @@ class RoutedMoE(nn.Module):
         a = torch.empty(E * T, ff, dtype=h.dtype, device=h.device)
         ops.clamp_glu(a, z[:, :ff], z[:, self.up_col: self.up_col + ff],
                       None, None, *self.glu)
-        y = torch.empty((E + 1) * T if self.shared is not None else E * T, W,
-                        dtype=h.dtype, device=h.device)
+        if self.shared is None:
+            y = torch.bmm(a.view(E, T, ff), self.w_down.transpose(1, 2))
+            ops.combine_rows_weighted(out, y.view(E * T, W), idx, wts)
+            return out
+        y = torch.empty((E + 1) * T, W, dtype=h.dtype, device=h.device)
         torch.bmm(a.view(E, T, ff), self.w_down.transpose(1, 2),
                   out=y[: E * T].view(E, T, W))
-        if self.shared is not None:
+        if True:
             self._shared_into(y[E * T:], h)
             idx[:, f.top] = self._arange(T, h.device) + E * T
             wts[:, f.top] = 1.0

@@ -23,6 +23,20 @@ def _pad8(n: int) -> int:
     return (n + 7) // 8 * 8
 
 
+def pad_rank(w1: torch.Tensor, w2: torch.Tensor, multiple: int = 16):
+    """A low-rank pair w2 f(w1 x) with f(0) = 0, its inner size brought up
+    to a multiple of `multiple` with zero rows of w1 and zero columns of w2:
+    the same function, and the first product is never narrower than the
+    matrix cores' tiles."""
+    n = -w1.shape[0] % multiple
+    if n:
+        w1 = torch.cat([w1, torch.zeros(n, w1.shape[1], dtype=w1.dtype,
+                                        device=w1.device)], 0)
+        w2 = torch.cat([w2, torch.zeros(w2.shape[0], n, dtype=w2.dtype,
+                                        device=w2.device)], 1)
+    return w1.contiguous(), w2.contiguous()
+
+
 def fuse_rows(segs, width: int, dtype, device):
     """Stack projection weights [rows_i, width] into one matrix whose
     segments each start on a multiple of 8 output columns.
@@ -492,10 +506,9 @@ class WkvMixer(nn.Module):
         self.w_rkvg = nn.Parameter(torch.stack(
             [t[p + n] for n in ("r", "k", "v", "g")]).to(**dev).contiguous(),
             requires_grad=False)
-        self.w1 = nn.Parameter(t[p + "w1"].to(**dev).contiguous(),
-                               requires_grad=False)
-        self.w2 = nn.Parameter(t[p + "w2"].to(**dev).contiguous(),
-                               requires_grad=False)
+        # the second, tiny product of the decay runs inside the scan (fp32)
+        w1, self.w2 = pad_rank(t[p + "w1"].to(**dev), t[p + "w2"].to(**f32))
+        self.w1 = nn.Parameter(w1, requires_grad=False)
         self.w0 = t[p + "w0"].to(**f32).contiguous()
         self.bonus = t[p + "u"].to(**f32).reshape(-1).contiguous()
         self.norm_w = t[p + "norm"].to(**f32).contiguous()
@@ -543,15 +556,19 @@ class WkvMixer(nn.Module):
         if not one:
             ops.token_shift_tail(prev, h, meta.positions, meta.cu_rows,
                                  meta.state_slots)
-        rkvg = torch.bmm(blends[:4], self.w_rkvg.transpose(1, 2))  # [4,T,C]
-        lo = ops.linear_f32(blends[4], self.w1)
-        lo_t = torch.empty(lo.shape, dtype=h.dtype, device=h.device)
-        ops.tanh_cast(lo_t, lo)
-        z = ops.linear_f32(lo_t, self.w2)                          # [T, C]
+        if T <= 64:
+            # decode steps: one batched product over the four blends
+            rkvg = torch.bmm(blends[:4], self.w_rkvg.transpose(1, 2))
+        else:
+            # prompt portions: four plain products into one buffer
+            rkvg = torch.empty(4, T, C, dtype=h.dtype, device=h.device)
+            for i in range(4):
+                torch.mm(blends[i], self.w_rkvg[i].t(), out=rkvg[i])
+        lo = ops.linear_f32(blends[4], self.w1)                    # [T, R]
         y = torch.empty(T, C, dtype=torch.float32, device=h.device)
-        ops.decay_scan(y, rkvg[0], rkvg[1], rkvg[2], z, self.w0, self.bonus,
-                       S, meta.positions, meta.cu_rows, meta.state_slots,
-                       m.heads, m.dim, m.dim, 0)
+        ops.decay_scan(y, rkvg[0], rkvg[1], rkvg[2], lo, self.w2, self.w0,
+                       self.bonus, S, meta.positions, meta.cu_rows,
+                       meta.state_slots, m.heads, m.dim, m.dim, 0)
         ops.head_rmsnorm_gate(out, y, rkvg[3], self.norm_w, m.heads,
                               self.eps, 0, scale)
 
@@ -702,11 +719,13 @@ class GatedLinearAttention(nn.Module):
         self.eps = eps
         self.col, self.w_in = fuse_rows(
             [("q", t[p + "q"]), ("k", t[p + "k"]), ("v", t[p + "v"]),
-             ("g", t[p + "g"]), ("a", t[p + "a1"])], width, dtype, device)
-        self.rank = t[p + "a1"].shape[0]
+             ("g", t[p + "g"])], width, dtype, device)
         f32 = dict(device=device, dtype=torch.float32)
-        self.w_a2 = nn.Parameter(t[p + "a2"].to(device=device, dtype=dtype)
-                                 .contiguous(), requires_grad=False)
+        # the decay's low-rank pair: the first product keeps its fp32 sums,
+        # the second, tiny one runs inside the scan
+        w1, self.w_a2 = pad_rank(t[p + "a1"].to(device=device, dtype=dtype),
+                                 t[p + "a2"].to(**f32))
+        self.w_a1 = nn.Parameter(w1, requires_grad=False)
         self.a_bias = t[p + "a2.b"].to(**f32).contiguous()
         self.norm_w = t[p + "norm"].to(**f32).repeat(m.heads).contiguous()
         self.w_o = nn.Parameter(t[p + "o"].to(device=device, dtype=dtype)
@@ -745,12 +764,12 @@ class GatedLinearAttention(nn.Module):
         c = self.col
         Cq, Cv = m.heads * m.dim, m.heads * m.vdim
         proj = ops.linear(h, self.w_in)
-        z = ops.linear_f32(proj[:, c["a"]: c["a"] + self.rank], self.w_a2)
+        lo = ops.linear_f32(h, self.w_a1)                          # [T, R]
         y = torch.empty(T, Cv, dtype=torch.float32, device=h.device)
         ops.decay_scan(y, proj[:, c["q"]: c["q"] + Cq],
                        proj[:, c["k"]: c["k"] + Cq],
-                       proj[:, c["v"]: c["v"] + Cv], z, self.a_bias, None,
-                       state, meta.positions, meta.cu_rows, meta.state_slots,
+                       proj[:, c["v"]: c["v"] + Cv], lo, self.w_a2,
+                       self.a_bias, None, state, meta.positions, meta.cu_rows, meta.state_slots,
                        m.heads, m.dim, m.vdim, 1, m.tau, m.dim ** -0.5)
         ops.head_rmsnorm_gate(out, y, proj[:, c["g"]: c["g"] + Cv],
                               self.norm_w, m.heads, self.eps, 0, scale)

@@ -769,14 +769,12 @@ def token_shift_tail(state, h, positions, cu_rows, state_slots) -> None:
     _strm(h).token_shift_tail(state, h, positions, cu_rows, state_slots)
 
 
-def tanh_cast(out, z) -> None:
-    _strm(out).tanh_cast(out, z)
-
-
-def decay_scan(y, q, k, v, z, zb, bonus, state, positions, cu_rows,
+def decay_scan(y, q, k, v, lo, w2, zb, bonus, state, positions, cu_rows,
                state_slots, H: int, d: int, dv: int, mode: int,
                tau: float = 1.0, q_scale: float = 1.0) -> None:
-    _strm(q).decay_scan(y, q, k, v, z, zb,
+    """Linear attention with a token-dependent decay per key channel whose
+    pre-activation is w2 f(lo) + zb (f = tanh in mode 0)."""
+    _strm(q).decay_scan(y, q, k, v, lo, w2, zb,
                         bonus if bonus is not None else _e(zb), state,
                         positions, cu_rows, state_slots, H, d, dv, mode, tau,
                         q_scale)

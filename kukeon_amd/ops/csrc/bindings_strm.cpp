@@ -22,15 +22,14 @@ void token_shift(torch::Tensor out, torch::Tensor h, torch::Tensor mu,
 void token_shift_tail(torch::Tensor state, torch::Tensor h,
                       torch::Tensor positions, torch::Tensor cu_rows,
                       torch::Tensor state_slots);
-void tanh_cast(torch::Tensor out, torch::Tensor z);
 void head_rmsnorm_gate(torch::Tensor out, torch::Tensor y, torch::Tensor gate,
                        torch::Tensor w, int64_t H, double eps, int64_t act,
                        double scale);
 void scaled_gate(torch::Tensor out, torch::Tensor a, torch::Tensor gate,
                  int64_t act, double scale);
 void decay_scan(torch::Tensor y, torch::Tensor q, torch::Tensor k,
-                torch::Tensor v, torch::Tensor z, torch::Tensor zb,
-                torch::Tensor bonus, torch::Tensor state,
+                torch::Tensor v, torch::Tensor lo, torch::Tensor w2,
+                torch::Tensor zb, torch::Tensor bonus, torch::Tensor state,
                 torch::Tensor positions, torch::Tensor cu_rows,
                 torch::Tensor state_slots, int64_t H, int64_t d, int64_t dv,
                 int64_t mode, double tau, double q_scale);
@@ -82,7 +81,6 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
         "out[n] = h + (row before - h) * mu[n], carried last row");
   m.def("token_shift_tail", &kukeon::token_shift_tail,
         "slot <- last row of a portion");
-  m.def("tanh_cast", &kukeon::tanh_cast, "tanh of fp32 rows");
   m.def("head_rmsnorm_gate", &kukeon::head_rmsnorm_gate,
         "per head y / rms(y) * w * act(gate) * scale");
   m.def("scaled_gate", &kukeon::scaled_gate, "a * act(gate) * scale");

@@ -5,8 +5,13 @@
 //           then S = diag(a_t) S + k_t v_t^T
 //   MODE 1  a_t = sigmoid(z_t + zb)^(1/tau);  S = diag(a_t) S + k_t v_t^T,
 //           then y_t = S^T (q_scale q_t)
-// z is the fp32 output of the decay's projection; the exponentials, the decay
-// and the whole recurrence are fp32. One workgroup per (sequence, head). The
+// The decay's pre-activation comes from a low-rank pair: z_t = W2 f(lo_t),
+// lo_t [R] being the fp32 output of the first projection (f = tanh in MODE 0,
+// the identity in MODE 1) and W2 [H d, R]; the second product is a handful
+// of multiply-adds per channel, so it is done here, in fp32, while a tile of
+// tokens is staged (the head's rows of W2 wait in LDS), and z never exists in
+// memory. The exponentials, the decay and the whole recurrence are fp32. One
+// workgroup per (sequence, head). The
 // state stays in registers for the whole portion: thread (e, l) owns the NR
 // consecutive key rows l NR .. l NR + NR - 1 of value column e, so a step is
 // a few fused multiply-adds per row plus a reduction over the LN neighbouring
@@ -30,7 +35,8 @@ template <typename T, int NR, int MODE>
 __global__ __launch_bounds__(1024) void decay_scan_kernel(
     float* __restrict__ y, const T* __restrict__ q, long ldq,
     const T* __restrict__ k, long ldk, const T* __restrict__ v, long ldv,
-    const float* __restrict__ z, long ldz, const float* __restrict__ zb,
+    const float* __restrict__ lo, long ldl, int R,
+    const float* __restrict__ w2, const float* __restrict__ zb,
     const float* __restrict__ bonus, float* __restrict__ state,
     const int* __restrict__ positions, const int* __restrict__ cu_rows,
     const int* __restrict__ state_slots, int H, int d, int dv, int LN,
@@ -41,6 +47,8 @@ __global__ __launch_bounds__(1024) void decay_scan_kernel(
   float* sK = sQ + DS_TT * DP;          // [TT][DP]
   float* sA = sK + DS_TT * DP;          // [TT][DP]
   float* sV = sA + DS_TT * DP;          // [TT][dv]
+  float* sLo = sV + DS_TT * dv;         // [TT][R]
+  float* sW2 = sLo + DS_TT * R;         // [d][R + 1]
   const int s = blockIdx.x;
   const int h = blockIdx.y;
   const long row0 = cu_rows[s];
@@ -54,6 +62,10 @@ __global__ __launch_bounds__(1024) void decay_scan_kernel(
     for (int i = tid; i < n * dv; i += nthreads)
       y[(row0 + i / dv) * (long)inner + h * dv + i % dv] = 0.f;
     return;
+  }
+  for (int i = tid; i < d * R; i += nthreads) {
+    const int dd = i / R, j = i - dd * R;
+    sW2[dd * (R + 1) + j] = w2[((long)h * d + dd) * R + j];
   }
   const int e = tid / LN;
   const int l = tid - e * LN;
@@ -87,6 +99,12 @@ __global__ __launch_bounds__(1024) void decay_scan_kernel(
   for (int t0 = 0; t0 < n; t0 += DS_TT) {
     const int nt = min(DS_TT, n - t0);
     __syncthreads();
+    for (int i = tid; i < nt * R; i += nthreads) {
+      const int t = i / R, j = i - t * R;
+      const float x = lo[(row0 + t0 + t) * ldl + j];
+      sLo[i] = MODE == 0 ? tanhf(x) : x;
+    }
+    __syncthreads();
     for (int i = tid; i < nt * DP; i += nthreads) {
       const int t = i / DP, dd = i - t * DP;
       const long r = row0 + t0 + t;
@@ -95,7 +113,9 @@ __global__ __launch_bounds__(1024) void decay_scan_kernel(
       if (dd < d) {
         qv = ldf(q + r * ldq + c) * q_scale;
         kv = ldf(k + r * ldk + c);
-        const float zz = z[r * ldz + c] + zb[c];
+        float zz = zb[c];
+        for (int j = 0; j < R; ++j)
+          zz = fmaf(sLo[t * R + j], sW2[dd * (R + 1) + j], zz);
         av = MODE == 0 ? expf(-expf(zz)) : expf(log_sigmoid(zz) * inv_tau);
       }
       sQ[i] = qv; sK[i] = kv; sA[i] = av;
@@ -160,11 +180,11 @@ __global__ __launch_bounds__(1024) void decay_scan_kernel(
 }
 
 // y [T, H*dv] fp32; q, k [T, H*d], v [T, H*dv] views (stride(1) == 1) in the
-// activation format; z [T, H*d] fp32 (stride(1) == 1); zb, bonus [H*d] fp32
-// (bonus empty in mode 1); state [slots, H, dv, d] fp32.
+// activation format; lo [T, R] fp32 (stride(1) == 1); w2 [H*d, R], zb, bonus
+// [H*d] fp32 (bonus empty in mode 1); state [slots, H, dv, d] fp32.
 void decay_scan(torch::Tensor y, torch::Tensor q, torch::Tensor k,
-                torch::Tensor v, torch::Tensor z, torch::Tensor zb,
-                torch::Tensor bonus, torch::Tensor state,
+                torch::Tensor v, torch::Tensor lo, torch::Tensor w2,
+                torch::Tensor zb, torch::Tensor bonus, torch::Tensor state,
                 torch::Tensor positions, torch::Tensor cu_rows,
                 torch::Tensor state_slots, int64_t H, int64_t d, int64_t dv,
                 int64_t mode, double tau, double q_scale) {
@@ -172,15 +192,18 @@ void decay_scan(torch::Tensor y, torch::Tensor q, torch::Tensor k,
   check_f32(y, "y"); check_f32(zb, "zb"); check_f32(state, "state");
   check_i32(positions, "positions"); check_i32(cu_rows, "cu_rows");
   check_i32(state_slots, "state_slots");
-  TORCH_CHECK(z.is_cuda() && z.scalar_type() == torch::kFloat32 &&
-              z.dim() == 2 && z.stride(1) == 1, "z must be fp32 rows");
+  TORCH_CHECK(lo.is_cuda() && lo.scalar_type() == torch::kFloat32 &&
+              lo.dim() == 2 && lo.stride(1) == 1, "lo must be fp32 rows");
+  check_f32(w2, "w2");
+  const int R = (int)lo.size(1);
+  TORCH_CHECK(R >= 1 && w2.dim() == 2 && w2.size(0) == H * d &&
+              w2.size(1) == R);
   TORCH_CHECK(mode == 0 || mode == 1);
   const long rows = q.size(0);
   TORCH_CHECK(q.dim() == 2 && k.dim() == 2 && v.dim() == 2 &&
               q.stride(1) == 1 && k.stride(1) == 1 && v.stride(1) == 1);
   TORCH_CHECK(q.size(1) == H * d && k.size(1) == H * d && v.size(1) == H * dv &&
-              k.size(0) == rows && v.size(0) == rows && z.size(0) == rows &&
-              z.size(1) == H * d);
+              k.size(0) == rows && v.size(0) == rows && lo.size(0) == rows);
   TORCH_CHECK(k.scalar_type() == q.scalar_type() &&
               v.scalar_type() == q.scalar_type());
   TORCH_CHECK(y.dim() == 2 && y.size(0) == rows && y.size(1) == H * dv);
@@ -208,15 +231,17 @@ void decay_scan(torch::Tensor y, torch::Tensor q, torch::Tensor k,
   const int need = (int)((d + LN - 1) / LN);
   const int NR = need <= 4 ? 4 : need <= 8 ? 8 : need <= 16 ? 16 : 32;
   const int threads = (int)((dv * LN + 63) / 64 * 64);
-  const size_t shmem = (size_t)DS_TT * (3 * LN * NR + dv) * sizeof(float);
+  const size_t shmem = ((size_t)DS_TT * (3 * LN * NR + dv + R) +
+                        (size_t)d * (R + 1)) * sizeof(float);
   TORCH_CHECK(shmem <= 64 * 1024, "head sizes exceed the staging buffers");
   auto stream = c10::hip::getCurrentHIPStream().stream();
   dim3 grid((unsigned)nseq, (unsigned)H);
 #define KK_ARGS y.data_ptr<float>(), reinterpret_cast<const T*>(q.data_ptr()),    \
         (long)q.stride(0), reinterpret_cast<const T*>(k.data_ptr()),              \
         (long)k.stride(0), reinterpret_cast<const T*>(v.data_ptr()),              \
-        (long)v.stride(0), z.data_ptr<float>(), (long)z.stride(0),                \
-        zb.data_ptr<float>(), mode == 0 ? bonus.data_ptr<float>() : nullptr,      \
+        (long)v.stride(0), lo.data_ptr<float>(), (long)lo.stride(0), R,           \
+        w2.data_ptr<float>(), zb.data_ptr<float>(),                               \
+        mode == 0 ? bonus.data_ptr<float>() : nullptr,                            \
         state.data_ptr<float>(), positions.data_ptr<int>(),                       \
         cu_rows.data_ptr<int>(), state_slots.data_ptr<int>(), (int)H, (int)d,     \
         (int)dv, LN, (float)(1.0 / (mode == 0 ? 1.0 : tau)), (float)q_scale

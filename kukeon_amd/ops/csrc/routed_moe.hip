@@ -72,11 +72,11 @@ void router_topk(torch::Tensor idx, torch::Tensor wts, torch::Tensor logits,
 // below the previous pick. A NaN logit counts as -inf.
 __global__ __launch_bounds__(256) void router_select_kernel(
     int* __restrict__ idx, float* __restrict__ wts, long ldi, long ldw,
-    const float* __restrict__ logits, long rows, int E, int top, int groups,
-    int keep, float scale, long dense_rows) {
+    const float* __restrict__ logits, long ldz, long rows, int E, int top,
+    int groups, int keep, float scale, long dense_rows) {
   const long t = (long)blockIdx.x * blockDim.x + threadIdx.x;
   if (t >= rows) return;
-  const float* z = logits + t * (long)E;
+  const float* z = logits + t * ldz;
   float vmax = -INFINITY;
   for (int e = 0; e < E; ++e) {
     const float v = z[e];
@@ -138,14 +138,17 @@ __global__ __launch_bounds__(256) void router_select_kernel(
 }
 
 // idx [T, >= top] int32, wts [T, >= top] fp32 (rows may be wider than top:
-// the other columns are left alone), logits [T, E] fp32.
+// the other columns are left alone), logits [T, E] fp32 (any row stride: the
+// first E columns of a wider product).
 void router_select(torch::Tensor idx, torch::Tensor wts, torch::Tensor logits,
                    int64_t top, int64_t groups, int64_t keep, double scale,
                    int64_t dense_rows) {
-  check_f32(logits, "logits");
+  TORCH_CHECK(logits.is_cuda() && logits.scalar_type() == torch::kFloat32 &&
+              logits.dim() == 2 && logits.stride(1) == 1,
+              "logits must be fp32 rows");
   TORCH_CHECK(idx.is_cuda() && idx.scalar_type() == torch::kInt32 &&
               wts.is_cuda() && wts.scalar_type() == torch::kFloat32);
-  TORCH_CHECK(logits.dim() == 2 && idx.dim() == 2 && wts.dim() == 2);
+  TORCH_CHECK(idx.dim() == 2 && wts.dim() == 2);
   const long rows = logits.size(0);
   const int E = (int)logits.size(1);
   TORCH_CHECK(top >= 1 && top <= E);
@@ -163,8 +166,9 @@ void router_select(torch::Tensor idx, torch::Tensor wts, torch::Tensor logits,
   router_select_kernel<<<dim3((unsigned)((rows + 255) / 256)), 256, 0,
                          stream>>>(
       idx.data_ptr<int>(), wts.data_ptr<float>(), (long)idx.stride(0),
-      (long)wts.stride(0), logits.data_ptr<float>(), rows, E, (int)top,
-      (int)groups, (int)keep, (float)scale, (long)dense_rows);
+      (long)wts.stride(0), logits.data_ptr<float>(), (long)logits.stride(0),
+      rows, E, (int)top, (int)groups, (int)keep, (float)scale,
+      (long)dense_rows);
   HIP_CHECK_KERNEL();
 }
 

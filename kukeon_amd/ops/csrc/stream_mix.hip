@@ -11,7 +11,6 @@
 //                            before a portion's first row is the sequence's
 //                            state slot (zeros at position 0)
 //   token_shift_tail         slot <- last row of a portion
-//   tanh_cast                fp32 -> tanh -> activation format
 //   head_rmsnorm_gate        per head y / rms(y) * w * act(gate) * scale
 //   scaled_gate              a * act(gate) * scale
 // One workgroup per row for the stream kernels; all arithmetic in fp32.
@@ -296,26 +295,6 @@ void token_shift_tail(torch::Tensor state, torch::Tensor h,
         state.data_ptr<float>(), reinterpret_cast<const T*>(h.data_ptr()),
         positions.data_ptr<int>(), cu_rows.data_ptr<int>(),
         state_slots.data_ptr<int>(), W);
-  });
-  HIP_CHECK_KERNEL();
-}
-
-template <typename T>
-__global__ __launch_bounds__(256) void tanh_cast_kernel(
-    T* __restrict__ out, const float* __restrict__ z, long n) {
-  const long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
-  if (i < n) stf(out + i, tanhf(z[i]));
-}
-
-void tanh_cast(torch::Tensor out, torch::Tensor z) {
-  check_act(out, "out"); check_f32(z, "z");
-  TORCH_CHECK(out.is_contiguous() && out.numel() == z.numel());
-  const long n = z.numel();
-  if (n == 0) return;
-  auto stream = c10::hip::getCurrentHIPStream().stream();
-  KK_DISPATCH_ACT(out, {
-    tanh_cast_kernel<T><<<dim3((unsigned)((n + 255) / 256)), 256, 0, stream>>>(
-        reinterpret_cast<T*>(out.data_ptr()), z.data_ptr<float>(), n);
   });
   HIP_CHECK_KERNEL();
 }

@@ -796,21 +796,21 @@ def token_shift_tail(state, h, positions, cu_rows, state_slots) -> None:
         state[int(state_slots[s])] = h[r1 - 1].float()
 
 
-def tanh_cast(out, z) -> None:
-    out.copy_(torch.tanh(z.float()).to(out.dtype))
-
-
-def decay_scan(y, q, k, v, z, zb, bonus, state, positions, cu_rows,
+def decay_scan(y, q, k, v, lo, w2, zb, bonus, state, positions, cu_rows,
                state_slots, H: int, d: int, dv: int, mode: int, tau: float,
                q_scale: float) -> None:
     """Linear attention with a decay per key channel, token after token.
-    Decay a_t = exp(-exp(z_t + zb)) (mode 0) or sigmoid(z_t + zb)^(1/tau)
-    (mode 1), fp32. Mode 0 reads before it writes and gives the current
+    The decay's pre-activation is z_t = w2 f(lo_t) + zb with lo [T, R] fp32,
+    w2 [H*d, R] and f = tanh (mode 0) or the identity (mode 1); the decay is
+    a_t = exp(-exp(z_t)) (mode 0) or sigmoid(z_t)^(1/tau) (mode 1), all
+    fp32. Mode 0 reads before it writes and gives the current
     token a bonus: y_t = (S + diag(bonus) k_t v_t^T)^T q_t, then
     S = diag(a_t) S + k_t v_t^T. Mode 1: S = diag(a_t) S + k_t v_t^T, then
     y_t = S^T (q_scale q_t). state [slots, H, dv, d] holds S^T (zeros at
     position 0); y [T, H*dv] fp32; q, k [T, H*d], v [T, H*dv] views."""
     nseq = cu_rows.numel() - 1
+    lof = lo.float()
+    z = (torch.tanh(lof) if mode == 0 else lof) @ w2.float().T + zb
     for s in range(nseq):
         r0, r1 = int(cu_rows[s]), int(cu_rows[s + 1])
         if r1 <= r0:
@@ -826,7 +826,7 @@ def decay_scan(y, q, k, v, z, zb, bonus, state, positions, cu_rows,
             qq = q[r].float().view(H, d) * q_scale
             kk = k[r].float().view(H, d)
             vv = v[r].float().view(H, dv)
-            zz = (z[r].float() + zb).view(H, d)
+            zz = z[r].view(H, d)
             kv = kk[:, :, None] * vv[:, None, :]
             if mode == 0:
                 a = torch.exp(-torch.exp(zz))

@@ -765,7 +765,11 @@ def case_op_scan(device, dtype, mode=0, H=3, d=5, dv=7, cuts=(4, 1, 9, 1, 1)):
     q = torch.randn(n, H * d, generator=g).to(act)
     k = (torch.randn(n, H * d, generator=g) * 0.5).to(act)
     v = torch.randn(n, H * dv, generator=g).to(act)
-    z = torch.randn(n, H * d, generator=g)
+    R = 3
+    lo = torch.randn(n, R, generator=g)
+    w2 = torch.randn(H * d, R, generator=g) * 0.6
+    z = (torch.tanh(lo.double()) if mode == 0 else lo.double()) @ \
+        w2.double().T
     zb = torch.randn(H * d, generator=g) - (1.0 if mode == 0 else -1.0)
     bonus = torch.randn(H * d, generator=g)
     tau, qs = 3.0, d ** -0.5 if mode else 1.0
@@ -796,8 +800,9 @@ def case_op_scan(device, dtype, mode=0, H=3, d=5, dv=7, cuts=(4, 1, 9, 1, 1)):
                                                            dtype=t.dtype)])
         pos, _, cu, slots = _maps([c, 2], [at, -1], device, [1, 0])
         y = torch.full((c + 2, H * dv), 5.0, device=device)
-        ops.decay_scan(y, dd(pad(q)), dd(pad(k)), dd(pad(v)), dd(pad(z)),
-                       dd(zb), dd(bonus) if mode == 0 else None, state, pos,
+        ops.decay_scan(y, dd(pad(q)), dd(pad(k)), dd(pad(v)), dd(pad(lo)),
+                       dd(w2), dd(zb), dd(bonus) if mode == 0 else None,
+                       state, pos,
                        cu, slots, H, d, dv, mode, tau, qs)
         assert float(y[c:].abs().max()) == 0.0
         got.append(y[:c])
@@ -945,3 +950,58 @@ def case_modelhub(device):
         c.close()
     finally:
         hub.stop()
+
+
+def case_real_sizes(device, say=lambda s: None):
+    """A stack at the layer sizes of a served model (heads of 128, pages of
+    16, rows of thousands of entries): the bf16 serving kernels against the
+    exact fp32 kernels, prompts on the packed path and decoding under
+    hipGraphs."""
+    from kukeon_amd.models.bezizen import bezizen_bench, random_tensors
+    mcfg = bezizen_bench(width=2048, layers=4, heads=16, kv_heads=4, ff=4096,
+                         vocab=512, window=96, experts=16, streams=4,
+                         max_positions=512, name="bezizen-sizes")
+    W = random_tensors(mcfg, 5)
+    g = torch.Generator().manual_seed(9)
+    prompts = [torch.randint(0, 512, (n,), generator=g).tolist()
+               for n in (150, 70, 129)]
+    outs = {}
+    for dtype in ("fp32", "bf16"):
+        say(f"model {dtype}")
+        model = BezizenModel(mcfg, device=device, dtype=dtype, tensors=W)
+        eng = LLMEngine(model, mcfg, EngineConfig(
+            block_size=16, max_model_len=512, max_sessions=4, state_slots=4,
+            num_kv_blocks=64, use_graphs=False), device=device)
+        say("prompts")
+        kvs = [SequenceKV(16) for _ in prompts]
+        lg = [eng.forward_tokens([(kv, p[:-6]) for kv, p in
+                                  zip(kvs, prompts)])]
+        say("single tokens")
+        for k in range(6, 0, -1):
+            lg.append(eng.forward_tokens([(kv, [p[-k]]) for kv, p in
+                                          zip(kvs, prompts)]))
+        outs[dtype] = torch.cat(lg).float().cpu()
+        assert bool(torch.isfinite(outs[dtype]).all())
+        for kv in kvs:
+            eng.free_sequence(kv)
+        if dtype == "bf16":
+            say("generation under graphs")
+            eng.ecfg.use_graphs = True
+            eng.ecfg.graph_buckets = (4,)
+            eng.ecfg.decode_microbatch = 8
+            sp = SamplingParams(temperature=0.7, top_k=50, top_p=0.9,
+                                max_new_tokens=17)
+            kvs = [SequenceKV(16) for _ in prompts]
+            rids = [eng.add_request(kv, p, sp) for kv, p in
+                    zip(kvs, prompts)]
+            n = 0
+            while eng.has_work():
+                for o in eng.step():
+                    n += len(o.new_tokens)
+                    assert all(0 <= t < 512 for t in o.new_tokens)
+            assert n == 17 * len(rids)
+        del eng, model
+    e = row_errors(outs["bf16"], outs["fp32"])
+    over = int((e > 0.15).sum())
+    assert over <= max(1, e.numel() // 4), f"{over} rows off, worst " \
+        f"{float(e.max()):.3g}"

@@ -130,3 +130,18 @@ def test_trace_runner(tmp_path):
 
 def test_modelhub_server():
     cases.case_modelhub(DEV)
+
+
+def test_bench_stack_shapes():
+    """The throughput stack at several sizes builds its configuration (no
+    weights): every layer has ff active rows, the last layer of a short stack
+    is a parallel one."""
+    from kukeon_amd.models.bezizen import bezizen_bench, tensor_shapes
+    for W, hq, hk, ff, nl in ((2048, 16, 4, 8192, 4), (8192, 64, 8, 28672, 2)):
+        cfg = bezizen_bench(width=W, layers=nl, heads=hq, kv_heads=hk, ff=ff,
+                            vocab=1000, max_positions=64)
+        assert cfg.layers[-1].type == "parallel"
+        for L in cfg.layers:
+            f = L.mlp
+            assert abs(f.shared_ff + f.top * f.ff - ff) <= 16
+        assert "l0.hc1.mix" in tensor_shapes(cfg)

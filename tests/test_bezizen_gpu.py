@@ -146,3 +146,9 @@ def test_trace_runner(tmp_path, dtype):
 
 def test_modelhub_server():
     cases.case_modelhub(DEV)
+
+
+def test_real_sizes():
+    def say(s):
+        print("real sizes:", s, flush=True)
+    cases.case_real_sizes(DEV, say)
