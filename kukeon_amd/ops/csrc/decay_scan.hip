@@ -10,7 +10,10 @@
 // the identity in MODE 1) and W2 [H d, R]; the second product is a handful
 // of multiply-adds per channel, so it is done here, in fp32, while a tile of
 // tokens is staged (the head's rows of W2 wait in LDS), and z never exists in
-// memory. The exponentials, the decay and the whole recurrence are fp32. One
+// memory. The bonus term of MODE 0 does not depend on the value column:
+// (diag(u) k v^T)^T q = v (sum_i u_i k_i q_i), so that sum is formed once per
+// token while the tile is staged and the inner loop keeps no copy of u. The
+// exponentials, the decay and the whole recurrence are fp32. One
 // workgroup per (sequence, head). The
 // state stays in registers for the whole portion: thread (e, l) owns the NR
 // consecutive key rows l NR .. l NR + NR - 1 of value column e, so a step is
@@ -49,6 +52,8 @@ __global__ __launch_bounds__(1024) void decay_scan_kernel(
   float* sV = sA + DS_TT * DP;          // [TT][dv]
   float* sLo = sV + DS_TT * dv;         // [TT][R]
   float* sW2 = sLo + DS_TT * R;         // [d][R + 1]
+  float* sU = sW2 + d * (R + 1);        // [d] bonus (MODE 0)
+  float* sC = sU + d;                   // [TT] sum_i u_i k_i q_i (MODE 0)
   const int s = blockIdx.x;
   const int h = blockIdx.y;
   const long row0 = cu_rows[s];
@@ -63,9 +68,35 @@ __global__ __launch_bounds__(1024) void decay_scan_kernel(
       y[(row0 + i / dv) * (long)inner + h * dv + i % dv] = 0.f;
     return;
   }
-  for (int i = tid; i < d * R; i += nthreads) {
-    const int dd = i / R, j = i - dd * R;
-    sW2[dd * (R + 1) + j] = w2[((long)h * d + dd) * R + j];
+  // A short portion (a decode step above all) is one dependent chain: the
+  // loads' completion is counted in issue order, so whatever is loaded after
+  // the state waits for the state. Its few inputs are therefore fetched into
+  // registers BEFORE the state loads are issued, and only committed to LDS
+  // afterwards; W2's rows likewise (up to four entries per thread).
+  const bool pre = n <= DS_TT && n * DP <= nthreads && n * dv <= nthreads &&
+                   n * R <= nthreads;
+  const bool prew = d * R <= 4 * nthreads;
+  float pw[4] = {0.f, 0.f, 0.f, 0.f};
+  float pq = 0.f, pk = 0.f, pv = 0.f, plo = 0.f, pu = 0.f;
+  if (prew) {
+#pragma unroll
+    for (int m = 0; m < 4; ++m) {
+      const int i = tid + m * nthreads;
+      if (i < d * R) pw[m] = w2[(long)h * d * R + i];
+    }
+  }
+  if (MODE == 0 && tid < d) pu = bonus[(long)h * d + tid];
+  if (pre) {
+    if (tid < n * DP) {
+      const int t = tid / DP, dd = tid - t * DP;
+      if (dd < d) {
+        pq = ldf(q + (row0 + t) * ldq + (long)h * d + dd);
+        pk = ldf(k + (row0 + t) * ldk + (long)h * d + dd);
+      }
+    }
+    if (tid < n * dv)
+      pv = ldf(v + (row0 + tid / dv) * ldv + (long)h * dv + tid % dv);
+    if (tid < n * R) plo = lo[(row0 + tid / R) * ldl + tid % R];
   }
   const int e = tid / LN;
   const int l = tid - e * LN;
@@ -73,7 +104,7 @@ __global__ __launch_bounds__(1024) void decay_scan_kernel(
   float* st = state + (((long)state_slots[s] * H + h) * dv + (live ? e : 0)) *
                           (long)d + l * NR;
   const bool vec4 = (d & 3) == 0;
-  float S[NR], U[MODE == 0 ? NR : 1];
+  float S[NR];
 #pragma unroll
   for (int i4 = 0; i4 < NR / 4; ++i4) {
     const int dd = l * NR + 4 * i4;
@@ -90,18 +121,28 @@ __global__ __launch_bounds__(1024) void decay_scan_kernel(
     }
     S[4 * i4 + 0] = sv.x; S[4 * i4 + 1] = sv.y;
     S[4 * i4 + 2] = sv.z; S[4 * i4 + 3] = sv.w;
-    if (MODE == 0) {
+  }
+  if (prew) {
 #pragma unroll
-      for (int j = 0; j < 4; ++j)
-        U[4 * i4 + j] = dd + j < d ? bonus[(long)h * d + dd + j] : 0.f;
+    for (int m = 0; m < 4; ++m) {
+      const int i = tid + m * nthreads;
+      if (i < d * R) sW2[(i / R) * (R + 1) + i % R] = pw[m];
     }
+  } else {
+    for (int i = tid; i < d * R; i += nthreads)
+      sW2[(i / R) * (R + 1) + i % R] = w2[(long)h * d * R + i];
+  }
+  if (MODE == 0) {
+    if (tid < d) sU[tid] = pu;
+    for (int i = tid + nthreads; i < d; i += nthreads)
+      sU[i] = bonus[(long)h * d + i];
   }
   for (int t0 = 0; t0 < n; t0 += DS_TT) {
     const int nt = min(DS_TT, n - t0);
     __syncthreads();
     for (int i = tid; i < nt * R; i += nthreads) {
       const int t = i / R, j = i - t * R;
-      const float x = lo[(row0 + t0 + t) * ldl + j];
+      const float x = pre ? plo : lo[(row0 + t0 + t) * ldl + j];
       sLo[i] = MODE == 0 ? tanhf(x) : x;
     }
     __syncthreads();
@@ -111,8 +152,8 @@ __global__ __launch_bounds__(1024) void decay_scan_kernel(
       const long c = (long)h * d + dd;
       float qv = 0.f, kv = 0.f, av = 0.f;
       if (dd < d) {
-        qv = ldf(q + r * ldq + c) * q_scale;
-        kv = ldf(k + r * ldk + c);
+        qv = (pre ? pq : ldf(q + r * ldq + c)) * q_scale;
+        kv = pre ? pk : ldf(k + r * ldk + c);
         float zz = zb[c];
         for (int j = 0; j < R; ++j)
           zz = fmaf(sLo[t * R + j], sW2[dd * (R + 1) + j], zz);
@@ -122,9 +163,22 @@ __global__ __launch_bounds__(1024) void decay_scan_kernel(
     }
     for (int i = tid; i < nt * dv; i += nthreads) {
       const int t = i / dv, ee = i - t * dv;
-      sV[i] = ldf(v + (row0 + t0 + t) * ldv + (long)h * dv + ee);
+      sV[i] = pre ? pv : ldf(v + (row0 + t0 + t) * ldv + (long)h * dv + ee);
     }
     __syncthreads();
+    if (MODE == 0) {
+      // 16 lanes per token share out the key channels
+      for (int i = tid; i < nt * 16; i += nthreads) {
+        const int t = i >> 4, part = i & 15;
+        float c = 0.f;
+        for (int dd = part; dd < d; dd += 16)
+          c = fmaf(sU[dd] * sK[t * DP + dd], sQ[t * DP + dd], c);
+#pragma unroll
+        for (int off = 8; off > 0; off >>= 1) c += __shfl_xor(c, off, WAVE);
+        if (part == 0) sC[t] = c;
+      }
+      __syncthreads();
+    }
     if (live) {
       for (int t = 0; t < nt; ++t) {
         const float vv = sV[t * dv + e];
@@ -148,7 +202,7 @@ __global__ __launch_bounds__(1024) void decay_scan_kernel(
           for (int j = 0; j < 4; ++j) {
             const float kvp = kk[j] * vv;
             if (MODE == 0) {
-              o = fmaf(fmaf(U[4 * i4 + j], kvp, Si[j]), q_[j], o);
+              o = fmaf(Si[j], q_[j], o);
               Si[j] = fmaf(aa[j], Si[j], kvp);
             } else {
               Si[j] = fmaf(aa[j], Si[j], kvp);
@@ -158,6 +212,7 @@ __global__ __launch_bounds__(1024) void decay_scan_kernel(
         }
         for (int off = LN >> 1; off > 0; off >>= 1)
           o += __shfl_xor(o, off, WAVE);
+        if (MODE == 0) o = fmaf(vv, sC[t], o);
         if (l == 0) y[(row0 + t0 + t) * (long)inner + h * dv + e] = o;
       }
     }
@@ -231,8 +286,8 @@ void decay_scan(torch::Tensor y, torch::Tensor q, torch::Tensor k,
   const int need = (int)((d + LN - 1) / LN);
   const int NR = need <= 4 ? 4 : need <= 8 ? 8 : need <= 16 ? 16 : 32;
   const int threads = (int)((dv * LN + 63) / 64 * 64);
-  const size_t shmem = ((size_t)DS_TT * (3 * LN * NR + dv + R) +
-                        (size_t)d * (R + 1)) * sizeof(float);
+  const size_t shmem = ((size_t)DS_TT * (3 * LN * NR + dv + R + 1) +
+                        (size_t)d * (R + 2)) * sizeof(float);
   TORCH_CHECK(shmem <= 64 * 1024, "head sizes exceed the staging buffers");
   auto stream = c10::hip::getCurrentHIPStream().stream();
   dim3 grid((unsigned)nseq, (unsigned)H);

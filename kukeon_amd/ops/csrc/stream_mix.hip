@@ -77,10 +77,32 @@ void embed_streams(torch::Tensor xs, torch::Tensor ids, torch::Tensor positions,
   HIP_CHECK_KERNEL();
 }
 
+// 4 consecutive elements in the storage format
+DEV_INLINE void ld4(const float* p, float* o) {
+  const float4 a = *reinterpret_cast<const float4*>(p);
+  o[0] = a.x; o[1] = a.y; o[2] = a.z; o[3] = a.w;
+}
+DEV_INLINE void ld4(const bf16_t* p, float* o) {
+  const uint2 a = *reinterpret_cast<const uint2*>(p);
+  o[0] = us2f((unsigned short)(a.x & 0xffffu)); o[1] = us2f((unsigned short)(a.x >> 16));
+  o[2] = us2f((unsigned short)(a.y & 0xffffu)); o[3] = us2f((unsigned short)(a.y >> 16));
+}
+DEV_INLINE void st4(float* p, const float* v) {
+  *reinterpret_cast<float4*>(p) = float4{v[0], v[1], v[2], v[3]};
+}
+DEV_INLINE void st4(bf16_t* p, const float* v) {
+  *reinterpret_cast<uint2*>(p) =
+      uint2{(unsigned)f2us(v[0]) | ((unsigned)f2us(v[1]) << 16),
+            (unsigned)f2us(v[2]) | ((unsigned)f2us(v[3]) << 16)};
+}
+
 // WRITE: first the streams' update from y, then the read. The blend u waits
-// in LDS (W floats) while the row's sum of squares is reduced.
-template <typename T, bool WRITE>
-__global__ __launch_bounds__(256) void stream_norm_kernel(
+// in LDS (W floats) while the row's sum of squares is reduced. V = 4: W is a
+// multiple of 4 and all rows 16-byte aligned, every access a 16-byte piece
+// (8 bytes for bf16); the workgroup is as wide as the row allows, so that a
+// step of few rows still has all of a row's loads in flight at once.
+template <typename T, bool WRITE, int V>
+__global__ __launch_bounds__(1024) void stream_norm_kernel(
     float* __restrict__ xs, const T* __restrict__ y, long ldy,
     const float* __restrict__ mix, const float* __restrict__ outc,
     const float* __restrict__ coef, const float* __restrict__ w, float eps,
@@ -98,38 +120,67 @@ __global__ __launch_bounds__(256) void stream_norm_kernel(
   float* xr = xs + r * (long)S * W;
   const T* yr = WRITE ? y + r * ldy : nullptr;
   float ss = 0.f;
-  for (int i = threadIdx.x; i < W; i += blockDim.x) {
-    float xo[SM_MAX_S];
+  for (int i = threadIdx.x * V; i < W; i += blockDim.x * V) {
+    float xo[SM_MAX_S][V];
 #pragma unroll
-    for (int s = 0; s < SM_MAX_S; ++s)
-      if (s < S) xo[s] = xr[(long)s * W + i];
-    float u = 0.f;
+    for (int s = 0; s < SM_MAX_S; ++s) {
+      if (s < S) {
+        if (V == 4) ld4(xr + (long)s * W + i, xo[s]);
+        else xo[s][0] = xr[(long)s * W + i];
+      }
+    }
+    float u[V];
+#pragma unroll
+    for (int k = 0; k < V; ++k) u[k] = 0.f;
     if (WRITE) {
-      const float yv = ldf(yr + i);
+      float yv[V];
+      if (V == 4) ld4(yr + i, yv);
+      else yv[0] = ldf(yr + i);
 #pragma unroll
       for (int j = 0; j < SM_MAX_S; ++j) {
         if (j < S) {
-          float v = 0.f;
+          float v[V];
 #pragma unroll
-          for (int s = 0; s < SM_MAX_S; ++s)
-            if (s < S) v = fmaf(smix[s * S + j], xo[s], v);
-          v = fmaf(sout[j], yv, v);
-          xr[(long)j * W + i] = v;
-          u = fmaf(scoef[j], v, u);
+          for (int k = 0; k < V; ++k) {
+            float a = 0.f;
+#pragma unroll
+            for (int s = 0; s < SM_MAX_S; ++s)
+              if (s < S) a = fmaf(smix[s * S + j], xo[s][k], a);
+            v[k] = fmaf(sout[j], yv[k], a);
+            u[k] = fmaf(scoef[j], v[k], u[k]);
+          }
+          if (V == 4) st4(xr + (long)j * W + i, v);
+          else xr[(long)j * W + i] = v[0];
         }
       }
     } else {
 #pragma unroll
       for (int s = 0; s < SM_MAX_S; ++s)
-        if (s < S) u = fmaf(scoef[s], xo[s], u);
+        if (s < S)
+#pragma unroll
+          for (int k = 0; k < V; ++k) u[k] = fmaf(scoef[s], xo[s][k], u[k]);
     }
-    su[i] = u;
-    ss = fmaf(u, u, ss);
+#pragma unroll
+    for (int k = 0; k < V; ++k) {
+      su[i + k] = u[k];
+      ss = fmaf(u[k], u[k], ss);
+    }
   }
   const float rs = 1.0f / sqrtf(block_sum2(ss, 0.f, red).x / (float)W + eps);
   T* orow = out + r * (long)W;
-  for (int i = threadIdx.x; i < W; i += blockDim.x)
-    stf(orow + i, su[i] * rs * w[i]);
+  for (int i = threadIdx.x * V; i < W; i += blockDim.x * V) {
+    float o[V];
+#pragma unroll
+    for (int k = 0; k < V; ++k) o[k] = su[i + k] * rs * w[i + k];
+    if (V == 4) st4(orow + i, o);
+    else stf(orow + i, o[0]);
+  }
+}
+
+// threads of a workgroup for rows of W entries taken V at a time
+static int stream_threads(int W, int V) {
+  const int want = (W / V + 63) / 64 * 64;
+  return want < 64 ? 64 : (want > 1024 ? 1024 : want);
 }
 
 static void stream_check(const torch::Tensor& xs, const torch::Tensor& coef,
@@ -153,20 +204,27 @@ void stream_read_norm(torch::Tensor out, torch::Tensor xs, torch::Tensor coef,
   if (rows == 0) return;
   auto stream = c10::hip::getCurrentHIPStream().stream();
   const size_t shmem = (size_t)(W + 32) * sizeof(float);
+  const bool vec = W % 4 == 0 && aligned16(xs.data_ptr()) &&
+                   aligned16(w.data_ptr()) && aligned16(out.data_ptr());
+#define KK_GO(V_)                                                             \
+  {                                                                           \
+    auto kern = stream_norm_kernel<T, false, V_>;                             \
+    static size_t allowed = 48 * 1024;                                        \
+    if (shmem > allowed) {                                                    \
+      hipFuncSetAttribute(reinterpret_cast<const void*>(kern),                \
+                          hipFuncAttributeMaxDynamicSharedMemorySize,         \
+                          (int)shmem);                                        \
+      allowed = shmem;                                                        \
+    }                                                                         \
+    kern<<<dim3((unsigned)rows), stream_threads(W, V_), shmem, stream>>>(     \
+        xs.data_ptr<float>(), nullptr, 0L, nullptr, nullptr,                  \
+        coef.data_ptr<float>(), w.data_ptr<float>(), (float)eps,              \
+        reinterpret_cast<T*>(out.data_ptr()), S, W);                          \
+  }
   KK_DISPATCH_ACT(out, {
-    auto kern = stream_norm_kernel<T, false>;
-    static size_t allowed = 48 * 1024;
-    if (shmem > allowed) {
-      hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                          hipFuncAttributeMaxDynamicSharedMemorySize,
-                          (int)shmem);
-      allowed = shmem;
-    }
-    kern<<<dim3((unsigned)rows), 256, shmem, stream>>>(
-        xs.data_ptr<float>(), nullptr, 0L, nullptr, nullptr,
-        coef.data_ptr<float>(), w.data_ptr<float>(), (float)eps,
-        reinterpret_cast<T*>(out.data_ptr()), S, W);
+    if (vec) KK_GO(4) else KK_GO(1)
   });
+#undef KK_GO
   HIP_CHECK_KERNEL();
 }
 
@@ -184,21 +242,29 @@ void stream_write_read_norm(torch::Tensor xs, torch::Tensor y,
   if (rows == 0) return;
   auto stream = c10::hip::getCurrentHIPStream().stream();
   const size_t shmem = (size_t)(W + 32) * sizeof(float);
+  const bool vec = W % 4 == 0 && y.stride(0) % 4 == 0 &&
+                   aligned16(xs.data_ptr()) && aligned16(w.data_ptr()) &&
+                   aligned16(out.data_ptr()) && aligned16(y.data_ptr());
+#define KK_GO(V_)                                                             \
+  {                                                                           \
+    auto kern = stream_norm_kernel<T, true, V_>;                              \
+    static size_t allowed = 48 * 1024;                                        \
+    if (shmem > allowed) {                                                    \
+      hipFuncSetAttribute(reinterpret_cast<const void*>(kern),                \
+                          hipFuncAttributeMaxDynamicSharedMemorySize,         \
+                          (int)shmem);                                        \
+      allowed = shmem;                                                        \
+    }                                                                         \
+    kern<<<dim3((unsigned)rows), stream_threads(W, V_), shmem, stream>>>(     \
+        xs.data_ptr<float>(), reinterpret_cast<const T*>(y.data_ptr()),       \
+        (long)y.stride(0), mix.data_ptr<float>(), outc.data_ptr<float>(),     \
+        coef.data_ptr<float>(), w.data_ptr<float>(), (float)eps,              \
+        reinterpret_cast<T*>(out.data_ptr()), S, W);                          \
+  }
   KK_DISPATCH_ACT(out, {
-    auto kern = stream_norm_kernel<T, true>;
-    static size_t allowed = 48 * 1024;
-    if (shmem > allowed) {
-      hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                          hipFuncAttributeMaxDynamicSharedMemorySize,
-                          (int)shmem);
-      allowed = shmem;
-    }
-    kern<<<dim3((unsigned)rows), 256, shmem, stream>>>(
-        xs.data_ptr<float>(), reinterpret_cast<const T*>(y.data_ptr()),
-        (long)y.stride(0), mix.data_ptr<float>(), outc.data_ptr<float>(),
-        coef.data_ptr<float>(), w.data_ptr<float>(), (float)eps,
-        reinterpret_cast<T*>(out.data_ptr()), S, W);
+    if (vec) KK_GO(4) else KK_GO(1)
   });
+#undef KK_GO
   HIP_CHECK_KERNEL();
 }
 
@@ -227,6 +293,41 @@ __global__ __launch_bounds__(256) void token_shift_kernel(
   if (shift) st[c] = cur;      // the sequence's only row: this thread's entry
 }
 
+// 8 consecutive entries per thread (W a multiple of 8, 16-byte aligned rows)
+template <typename T>
+__global__ __launch_bounds__(256) void token_shift_vec_kernel(
+    T* __restrict__ out, const T* __restrict__ h, const float* __restrict__ mu,
+    float* __restrict__ state, const int* __restrict__ positions,
+    const int* __restrict__ row_seq, const int* __restrict__ cu_rows,
+    const int* __restrict__ state_slots, long rows, int N, int W, int shift) {
+  const long r = blockIdx.x;
+  const int c = (blockIdx.y * blockDim.x + threadIdx.x) * 8;
+  if (c >= W) return;
+  const int p = positions[r];
+  if (p < 0) return;
+  const int s = row_seq[r];
+  const long row0 = cu_rows[s];
+  float* st = state + (long)state_slots[s] * W;
+  float cur[8], prev[8];
+  ld8(h + r * (long)W + c, cur);
+  if (r > row0) {
+    ld8(h + (r - 1) * (long)W + c, prev);
+  } else if (p > 0) {
+    ld8(st + c, prev);
+  } else {
+#pragma unroll
+    for (int k = 0; k < 8; ++k) prev[k] = 0.f;
+  }
+  for (int n = 0; n < N; ++n) {
+    float m[8], o[8];
+    ld8(mu + (long)n * W + c, m);
+#pragma unroll
+    for (int k = 0; k < 8; ++k) o[k] = fmaf(prev[k] - cur[k], m[k], cur[k]);
+    st8(out + ((long)n * rows + r) * W + c, o);
+  }
+  if (shift) st8(st + c, cur);
+}
+
 void token_shift(torch::Tensor out, torch::Tensor h, torch::Tensor mu,
                  torch::Tensor state, torch::Tensor positions,
                  torch::Tensor row_seq, torch::Tensor cu_rows,
@@ -249,15 +350,25 @@ void token_shift(torch::Tensor out, torch::Tensor h, torch::Tensor mu,
               "the slot is shifted in place only when every sequence brings "
               "one row");
   auto stream = c10::hip::getCurrentHIPStream().stream();
-  dim3 grid((unsigned)rows, (unsigned)((W + 255) / 256));
+  const bool vec = W % 8 == 0 && aligned16(out.data_ptr()) &&
+                   aligned16(h.data_ptr()) && aligned16(mu.data_ptr()) &&
+                   aligned16(state.data_ptr());
+#define KK_ARGS reinterpret_cast<T*>(out.data_ptr()),                          \
+        reinterpret_cast<const T*>(h.data_ptr()), mu.data_ptr<float>(),       \
+        state.data_ptr<float>(), positions.data_ptr<int>(),                   \
+        row_seq.data_ptr<int>(), cu_rows.data_ptr<int>(),                     \
+        state_slots.data_ptr<int>(), rows, N, W, (int)shift_state
   KK_DISPATCH_ACT(h, {
-    token_shift_kernel<T><<<grid, 256, 0, stream>>>(
-        reinterpret_cast<T*>(out.data_ptr()),
-        reinterpret_cast<const T*>(h.data_ptr()), mu.data_ptr<float>(),
-        state.data_ptr<float>(), positions.data_ptr<int>(),
-        row_seq.data_ptr<int>(), cu_rows.data_ptr<int>(),
-        state_slots.data_ptr<int>(), rows, N, W, (int)shift_state);
+    if (vec) {
+      const int threads = W / 8 >= 256 ? 256 : 64;
+      dim3 grid((unsigned)rows, (unsigned)((W / 8 + threads - 1) / threads));
+      token_shift_vec_kernel<T><<<grid, threads, 0, stream>>>(KK_ARGS);
+    } else {
+      dim3 grid((unsigned)rows, (unsigned)((W + 255) / 256));
+      token_shift_kernel<T><<<grid, 256, 0, stream>>>(KK_ARGS);
+    }
   });
+#undef KK_ARGS
   HIP_CHECK_KERNEL();
 }
 
@@ -321,6 +432,36 @@ __global__ __launch_bounds__(256) void head_rmsnorm_gate_kernel(
         yr[i] * rs * w[c0 + i] * gate_act(ldf(gate + r * ldg + c0 + i), act));
 }
 
+// LPH = dv / 8 lanes per (row, head), 8 consecutive entries per lane; the sum
+// of squares meets over the LPH neighbouring lanes.
+template <typename T>
+__global__ __launch_bounds__(256) void head_rmsnorm_gate_vec_kernel(
+    T* __restrict__ out, long ldo, const float* __restrict__ y,
+    const T* __restrict__ gate, long ldg, const float* __restrict__ w, long rows,
+    int H, int dv, int LPH, float eps, int act, float scale) {
+  const long t = (long)blockIdx.x * blockDim.x + threadIdx.x;
+  const long unit = t / LPH;
+  const int sub = (int)(t - unit * LPH);
+  const bool live = unit < rows * H;
+  const long r = live ? unit / H : 0;
+  const int hd = live ? (int)(unit - r * H) : 0;
+  const long c0 = (long)hd * dv + sub * 8;
+  float v[8];
+  ld8(y + r * (long)H * dv + c0, v);
+  float ss = 0.f;
+#pragma unroll
+  for (int k = 0; k < 8; ++k) ss = fmaf(v[k], v[k], ss);
+  for (int off = LPH >> 1; off > 0; off >>= 1) ss += __shfl_xor(ss, off, WAVE);
+  if (!live) return;
+  const float rs = scale / sqrtf(ss / (float)dv + eps);
+  float g[8], ww[8], o[8];
+  ld8(gate + r * ldg + c0, g);
+  ld8(w + c0, ww);
+#pragma unroll
+  for (int k = 0; k < 8; ++k) o[k] = v[k] * rs * ww[k] * gate_act(g[k], act);
+  st8(out + r * ldo + c0, o);
+}
+
 void head_rmsnorm_gate(torch::Tensor out, torch::Tensor y, torch::Tensor gate,
                        torch::Tensor w, int64_t H, double eps, int64_t act,
                        double scale) {
@@ -336,6 +477,25 @@ void head_rmsnorm_gate(torch::Tensor out, torch::Tensor y, torch::Tensor gate,
   if (rows == 0) return;
   auto stream = c10::hip::getCurrentHIPStream().stream();
   const long units = rows * H;
+  const int dvh = (int)(C / H);
+  const int LPH = dvh / 8;
+  const bool vec = dvh % 8 == 0 && LPH <= WAVE && (LPH & (LPH - 1)) == 0 &&
+                   out.stride(0) % 8 == 0 && gate.stride(0) % 8 == 0 &&
+                   aligned16(out.data_ptr()) && aligned16(y.data_ptr()) &&
+                   aligned16(gate.data_ptr()) && aligned16(w.data_ptr());
+  if (vec) {
+    const long threads = units * LPH;
+    KK_DISPATCH_ACT(out, {
+      head_rmsnorm_gate_vec_kernel<T><<<dim3((unsigned)((threads + 255) / 256)),
+                                        256, 0, stream>>>(
+          reinterpret_cast<T*>(out.data_ptr()), (long)out.stride(0),
+          y.data_ptr<float>(), reinterpret_cast<const T*>(gate.data_ptr()),
+          (long)gate.stride(0), w.data_ptr<float>(), rows, (int)H, dvh, LPH,
+          (float)eps, (int)act, (float)scale);
+    });
+    HIP_CHECK_KERNEL();
+    return;
+  }
   KK_DISPATCH_ACT(out, {
     head_rmsnorm_gate_kernel<T><<<dim3((unsigned)((units + 3) / 4)), 256, 0,
                                   stream>>>(
