@@ -502,7 +502,7 @@ class WkvMixer(nn.Module):
         dev = dict(device=device, dtype=dtype)
         self.mu = torch.stack([t[p + "mu." + n] for n in self.BLENDS]).to(
             **f32).contiguous()
-        # r, k, v, g have one shape: one batched GEMM over their blends
+        # r, k, v, g have one shape: their matrices are kept stacked
         self.w_rkvg = nn.Parameter(torch.stack(
             [t[p + n] for n in ("r", "k", "v", "g")]).to(**dev).contiguous(),
             requires_grad=False)
@@ -556,14 +556,10 @@ class WkvMixer(nn.Module):
         if not one:
             ops.token_shift_tail(prev, h, meta.positions, meta.cu_rows,
                                  meta.state_slots)
-        if T <= 64:
-            # decode steps: one batched product over the four blends
-            rkvg = torch.bmm(blends[:4], self.w_rkvg.transpose(1, 2))
-        else:
-            # prompt portions: four plain products into one buffer
-            rkvg = torch.empty(4, T, C, dtype=h.dtype, device=h.device)
-            for i in range(4):
-                torch.mm(blends[i], self.w_rkvg[i].t(), out=rkvg[i])
+        # four plain products into one buffer (each blend has its own matrix)
+        rkvg = torch.empty(4, T, C, dtype=h.dtype, device=h.device)
+        for i in range(4):
+            torch.mm(blends[i], self.w_rkvg[i].t(), out=rkvg[i])
         lo = ops.linear_f32(blends[4], self.w1)                    # [T, R]
         y = torch.empty(T, C, dtype=torch.float32, device=h.device)
         ops.decay_scan(y, rkvg[0], rkvg[1], rkvg[2], lo, self.w2, self.w0,
