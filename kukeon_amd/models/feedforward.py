@@ -334,10 +334,9 @@ class RoutedMoE(nn.Module):
         y = torch.empty((E + 1) * T, W, dtype=h.dtype, device=h.device)
         torch.bmm(a.view(E, T, ff), self.w_down.transpose(1, 2),
                   out=y[: E * T].view(E, T, W))
-        if True:
-            self._shared_into(y[E * T:], h)
-            idx[:, f.top] = self._arange(T, h.device) + E * T
-            wts[:, f.top] = 1.0
+        self._shared_into(y[E * T:], h)
+        idx[:, f.top] = self._arange(T, h.device) + E * T
+        wts[:, f.top] = 1.0
         ops.combine_rows_weighted(out, y, idx, wts)
         return out
 

@@ -635,7 +635,6 @@ def case_router(device, dtype):
     """Routed experts alone against the plain model: groups, every `top`,
     rows in both forms of the expert pass."""
     from kukeon_amd.models.feedforward import FFCfg, RoutedMoE
-    from kukeon_amd.engine.config import ModelConfig  # noqa: F401
     Wd = 24
     for E, top, groups, shared, T in ((6, 2, (3, 2), 8, 5), (8, 3, (2, 1), 0, 70),
                                       (4, 4, None, 6, 66), (5, 1, None, 0, 3)):
